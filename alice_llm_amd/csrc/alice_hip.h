@@ -4,11 +4,13 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define ALICE_ABI_VERSION 9
+#define ALICE_ABI_VERSION 10
 
 #define ALICE_EPI_NONE 0
 #define ALICE_EPI_GEGLU 1     // W = [gate; up] stacked; epi_param 0: y = gelu_tanh(gate x) * (up x); epi_param = limit > 0:
-                              // g = min(gate x, limit), u = clamp(up x, -limit, limit), y = g * sigmoid(1.702 g) * (u + 1)
+                              // g = min(gate x, limit), u = clamp(up x, -limit, limit), y = g * sigmoid(1.702 g) * (u + 1);
+                              // ALICE_GATED_SILU: y = (gate x) * sigmoid(gate x) * (up x)
+#define ALICE_GATED_SILU (-1.0f)
 #define ALICE_EPI_SOFTCAP 2   // one function of each output element, its form picked by epi_param: cap > 0: y = cap * tanh(y / cap);
                               // ALICE_UNARY_RELU2: y = max(y, 0)^2
 #define ALICE_UNARY_RELU2 (-1.0f)
@@ -162,6 +164,22 @@ int alice_gla(const float* rows, int row_w, int q_col, int k_col, int v_col, int
               const float* z_bias, float tau, float q_scale, float out_scale, const void* norm_w, int w_dtype, float eps, void* out,
               int out_dtype, float* work, const int* cu_seqlens, const int* slots, float* S, int T, int n_seqs,
               int n_slots, int H, int d, int dv, int columns, hipStream_t stream);
+// Latent attention (latent.hip): the cache row of a token is [latent (kv_rank) | rotated key part (rot_dim)], one kv head,
+// row-major pages; the first kv_rank dimensions of a row are also its value.
+int alice_latent_prepare(const float* rows, int row_width, int q_rank, int kv_rank, int rot_dim, const float* w_q,
+                         const float* w_kv, float eps, const float* cos_t, const float* sin_t, const int* positions,
+                         const int* seq_of_token, const int* block_table, int bt_stride, int page_size, int n_pages,
+                         void* q_latent, void* k_pool, int out_dtype, int T, hipStream_t stream);
+// y[t, h, 0:n] = M_h x[t, h, 0:k], M transposed [H, k, n]; y[t, h, n:n+rot_dim] = x[t, h, k:k+rot_dim] rotated in pairs
+// (2i, 2i + 1) by the token's position (tables [positions, rot_dim / 2]).  Rows and heads by their strides in elements.
+int alice_heads_linear(const void* x, int x_dtype, long x_row, int x_head, const void* wt, int w_dtype, void* y,
+                       int y_dtype, long y_row, int y_head, int T, int H, int n, int k, int rot_dim, const float* cos_t,
+                       const float* sin_t, const int* positions, hipStream_t stream);
+// q [T, nH, kv_rank + rot_dim] against the cached rows of the token's sequence: keys max(0, pos + 1 - window) .. pos
+// (window 0: all), softmax of scale * q.k, out [T, nH, kv_rank] = weights times the rows' first kv_rank dimensions.
+int alice_latent_attention(const void* q, int dtype, const void* k_pool, void* out, const int* positions,
+                           const int* seq_of_token, const int* block_table, int bt_stride, int T, int nH, int kv_rank,
+                           int rot_dim, int page_size, float scale, int window, int full_precision, hipStream_t stream);
 int alice_head_gate(void* out, int out_layout, const void* gate, int gate_stride, int T, int nH, int d, hipStream_t stream);
 long alice_attention_decode_workspace(int B, int nH, int d, int splits);
 // out may be absent when splits > 1: the splits are then left in `parts`, [B][nH][splits][ALICE_ATTN_PARTS_HEAD + d]

@@ -104,8 +104,13 @@ __device__ __forceinline__ float gelu_tanh_f(float z, bool full) {
 
 // The gated product of two stacked matrices' outputs (gate g, up u), the epilogue ALICE_EPI_GEGLU.  Its
 // parameter picks the form: 0 gives gelu_tanh(g) * u; a positive `limit` gives the limited form
-// g' = min(g, limit), u' = clamp(u, -limit, limit), g' * sigmoid(1.702 g') * (u' + 1).
+// g' = min(g, limit), u' = clamp(u, -limit, limit), g' * sigmoid(1.702 g') * (u' + 1); a negative one
+// (ALICE_GATED_SILU) gives g * sigmoid(g) * u.
 __device__ __forceinline__ float gated_act(float g, float u, float limit, bool full) {
+  if (limit < 0.f) {
+    const float e = full ? expf(-g) : __expf(-g);
+    return g / (1.f + e) * u;
+  }
   if (limit > 0.f) {
     g = fminf(g, limit);
     u = fminf(fmaxf(u, -limit), limit);

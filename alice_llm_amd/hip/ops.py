@@ -18,7 +18,8 @@ from ..csrc import build as _build
 EPI_NONE, EPI_GEGLU, EPI_SOFTCAP = 0, 1, 2
 LAYOUT_ROW, LAYOUT_FRAG16 = 0, 1
 LINEAR_AUTO, LINEAR_GENERIC, LINEAR_SKINNY, LINEAR_MFMA, LINEAR_TILED_W16, LINEAR_TILED_W32 = 0, 1, 2, 3, 4, 5
-ABI_VERSION = 9
+ABI_VERSION = 10
+GATED_SILU = -1.0        # epi_param of EPI_GEGLU that picks silu(gate) * up
 UNARY_RELU2 = -1.0       # epi_param of EPI_SOFTCAP that picks the square of max(y, 0) instead of the capped form
 
 _lib = None
@@ -66,6 +67,9 @@ def _declare(lib) -> None:
         "alice_mix_heads": [P, P, P, I, F, P, I, I, I, I, I, I, P],
         "alice_qkv_prepare": [P, I, I, P, P, P, P, I, P, P, I, I, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
         "alice_add_rows": [P, P, P, I, I, P],
+        "alice_latent_prepare": [P, I, I, I, I, P, P, F, P, P, P, P, P, I, I, I, P, P, I, I, P],
+        "alice_heads_linear": [P, I, L, I, P, I, P, I, L, I, I, I, I, I, I, P, P, P, P],
+        "alice_latent_attention": [P, I, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
         "alice_gla": [P, I, I, I, I, I, P, P, F, F, F, P, I, F, P, I, P, P, P, P, I, I, I, I, I, I, I, P],
         "alice_linear_parts_split": [I, I, I, I, I],
         "alice_linear_parts": [P, I, I, I, P, P, I, I, P],
@@ -749,6 +753,100 @@ def add_rows(x: torch.Tensor, rows: Optional[torch.Tensor], vector: Optional[tor
     _dev(x, "x", torch.float32)
     _call("alice_add_rows", x.data_ptr(), _opt(rows, "rows", torch.float32, (T, W)), _opt(vector, "vector", torch.float32, (W,)),
           T, W, _stream())
+
+
+
+# ------------------------------------------------------------------------------------ latent attention
+
+LATENT_MAX_RANK = 1024       # the largest latent the latent attention kernels take
+
+
+def _latent_pool(k_pool: torch.Tensor, kv_rank: int, rot_dim: int, dt) -> None:
+    if k_pool.dim() != 4 or k_pool.shape[1] != 1 or k_pool.shape[3] != kv_rank + rot_dim:
+        raise HipLibraryError(f"k_pool must be [pages, 1, page, {kv_rank + rot_dim}], found {tuple(k_pool.shape)}")
+    _dev(k_pool, "k_pool", dt)
+
+
+def _rot_tables(cos, sin, rot_dim: int, max_position: int):
+    if rot_dim == 0:
+        return None, None
+    if cos is None or sin is None or cos.dim() != 2 or cos.shape[1] != rot_dim // 2 or sin.shape != cos.shape or rot_dim % 2:
+        raise HipLibraryError(f"cos/sin must be [positions, {rot_dim // 2}]")
+    if max_position >= cos.shape[0]:
+        raise HipLibraryError(f"position {max_position} is beyond the rotation tables ({cos.shape[0]} positions)")
+    return _dev(cos, "cos", torch.float32), _dev(sin, "sin", torch.float32)
+
+
+def latent_prepare(rows: torch.Tensor, w_q: torch.Tensor, w_kv: torch.Tensor, q_latent: torch.Tensor,
+                   k_pool: Optional[torch.Tensor], positions: torch.Tensor, seq_of_token: Optional[torch.Tensor],
+                   block_table: Optional[torch.Tensor], *, q_rank: int, kv_rank: int, rot_dim: int, eps: float,
+                   cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], max_position: int) -> None:
+    """From the float32 rows [a (q_rank) | c (kv_rank) | kr (rot_dim)] of a fused down projection: the RMS-normed a
+    (weight w_q) to q_latent [T, q_rank]; the RMS-normed c (weight w_kv) and kr rotated in pairs (2i, 2i + 1) into the
+    token's row of the cache, [pages, 1, page, kv_rank + rot_dim] (None: nothing is cached)."""
+    T = rows.shape[0]
+    if rows.dim() != 2 or rows.shape[1] < q_rank + kv_rank + rot_dim:
+        raise HipLibraryError(f"rows must be [T, >= {q_rank + kv_rank + rot_dim}], found {tuple(rows.shape)}")
+    _dev(rows, "rows", torch.float32)
+    _dev(w_q, "w_q", torch.float32, (q_rank,))
+    _dev(w_kv, "w_kv", torch.float32, (kv_rank,))
+    _dev(q_latent, "q_latent", None, (T, q_rank))
+    _dev(positions, "positions", torch.int32, (T,))
+    c, s_ = _rot_tables(cos, sin, rot_dim, max_position)
+    page_size = n_pages = bt_stride = 0
+    if k_pool is not None:
+        _latent_pool(k_pool, kv_rank, rot_dim, q_latent.dtype)
+        n_pages, _, page_size, _ = k_pool.shape
+        _dev(seq_of_token, "seq_of_token", torch.int32, (T,))
+        _dev(block_table, "block_table", torch.int32)
+        if block_table.dim() != 2 or max_position // page_size >= block_table.shape[1]:
+            raise HipLibraryError(f"position {max_position} is beyond the block table")
+        bt_stride = block_table.shape[1]
+    _call("alice_latent_prepare", rows.data_ptr(), rows.shape[1], q_rank, kv_rank, rot_dim, w_q.data_ptr(), w_kv.data_ptr(),
+          float(eps), c, s_, positions.data_ptr(), _opt(seq_of_token, "seq_of_token"), _opt(block_table, "block_table"),
+          bt_stride, page_size, n_pages, q_latent.data_ptr(), _opt(k_pool, "k_pool"), dtype_code(q_latent.dtype), T, _stream())
+
+
+def heads_linear(x: torch.Tensor, wt: torch.Tensor, y: torch.Tensor, *, heads: int, n: int, k: int, rot_dim: int = 0,
+                 cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
+                 positions: Optional[torch.Tensor] = None, max_position: int = 0) -> None:
+    """A matrix a head: y[t, h, 0:n] = M_h x[t, h, 0:k] with M given transposed, wt [heads, k, n]; x [T, heads * (k +
+    rot_dim)], y [T, heads * (n + rot_dim)]; the rot_dim elements behind a head's k inputs are rotated in pairs
+    (2i, 2i + 1) by the token's position and put behind its n outputs."""
+    T = x.shape[0]
+    _dev(x, "x", None, (T, heads * (k + rot_dim)))
+    _dev(y, "y", None, (T, heads * (n + rot_dim)))
+    _dev(wt, "wt", None, (heads, k, n))
+    c, s_ = _rot_tables(cos, sin, rot_dim, max_position)
+    if rot_dim:
+        _dev(positions, "positions", torch.int32, (T,))
+    _call("alice_heads_linear", x.data_ptr(), dtype_code(x.dtype), heads * (k + rot_dim), k + rot_dim, wt.data_ptr(),
+          dtype_code(wt.dtype), y.data_ptr(), dtype_code(y.dtype), heads * (n + rot_dim), n + rot_dim, T, heads, n, k,
+          rot_dim, c, s_, positions.data_ptr() if rot_dim else None, _stream())
+
+
+def latent_attention(q: torch.Tensor, k_pool: torch.Tensor, out: torch.Tensor, ctx, block_table: torch.Tensor, *,
+                     num_heads: int, kv_rank: int, rot_dim: int, scale: float, window: Optional[int],
+                     full_precision: bool) -> None:
+    """Softmax attention of q [T, heads * (kv_rank + rot_dim)] over the cached rows [latent | rotated part] of each
+    token's sequence, keys max(0, pos + 1 - window) .. pos; out [T, heads * kv_rank] = the weights times the rows'
+    latents.  32-bit arithmetic, any sizes up to LATENT_MAX_RANK."""
+    T = q.shape[0]
+    dt = q.dtype
+    _latent_pool(k_pool, kv_rank, rot_dim, dt)
+    if not 1 <= kv_rank <= LATENT_MAX_RANK:
+        raise HipLibraryError(f"latent size {kv_rank} is outside 1..{LATENT_MAX_RANK}")
+    _dev(q, "q", None, (T, num_heads * (kv_rank + rot_dim)))
+    _dev(out, "out", dt, (T, num_heads * kv_rank))
+    _dev(ctx.positions, "positions", torch.int32, (T,))
+    _dev(ctx.seq_of_token, "seq_of_token", torch.int32, (T,))
+    _dev(block_table, "block_table", torch.int32)
+    page_size = k_pool.shape[2]
+    if block_table.dim() != 2 or ctx.max_position // page_size >= block_table.shape[1] or block_table.shape[0] < ctx.n_seqs:
+        raise HipLibraryError(f"position {ctx.max_position} is beyond the block table")
+    _call("alice_latent_attention", q.data_ptr(), dtype_code(dt), k_pool.data_ptr(), out.data_ptr(), ctx.positions.data_ptr(),
+          ctx.seq_of_token.data_ptr(), block_table.data_ptr(), block_table.shape[1], T, num_heads, kv_rank, rot_dim, page_size,
+          float(scale), int(window or 0), int(full_precision), _stream())
 
 
 GLA_MAX_KEY_DIM = 256       # the largest key size the gated linear attention kernel keeps in registers

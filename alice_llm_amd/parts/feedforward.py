@@ -1,7 +1,8 @@
 """Feed-forwards.  Gated MLP: down( act(gate x) * (up x) ), the activation on the gate branch
 (llama3.rs:14519-14540); for Gemma 2 the activation is the tanh form of GELU
 (llama3.rs:6183-6186).  A second gated form, "swish_limited", bounds both branches first:
-g = min(gate x, limit), u = clamp(up x, -limit, limit), y = g * sigmoid(1.702 g) * (u + 1).  gate and up are stacked into one matrix at load so that one kernel reads
+g = min(gate x, limit), u = clamp(up x, -limit, limit), y = g * sigmoid(1.702 g) * (u + 1); a third, "silu", is
+silu(gate x) * (up x) with silu(z) = z * sigmoid(z).  gate and up are stacked into one matrix at load so that one kernel reads
 the input once and applies the activation and the product in its epilogue.
 
 Dense MLP: down( act(up x) ), the activation as the epilogue of the first product; "relu_squared" is
@@ -18,8 +19,8 @@ from .base import FEED_FORWARDS, ParamSpec, Part, Precision
 from .linear import Linear
 
 # both forms are the gated epilogue of the matrix products; its parameter picks the form (0: tanh-GELU times up;
-# a positive limit: the limited swish form)
-_GATED_EPILOGUES = {"gelu_tanh": ops.EPI_GEGLU, "swish_limited": ops.EPI_GEGLU}
+# a positive limit: the limited swish form; ops.GATED_SILU: silu times up)
+_GATED_EPILOGUES = {"gelu_tanh": ops.EPI_GEGLU, "swish_limited": ops.EPI_GEGLU, "silu": ops.EPI_GEGLU}
 _DEFAULT_NAMES = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
 
 
@@ -38,7 +39,7 @@ class GatedMLP(Part):
         self.H, self.I = hidden_size, intermediate_size
         self.names = dict(_DEFAULT_NAMES, **(tensor_names or {}))
         self.gate_up = Linear(hidden_size, intermediate_size, precision, epilogue=_GATED_EPILOGUES[activation],
-                              epi_param=float(limit or 0.0))
+                              epi_param=ops.GATED_SILU if activation == "silu" else float(limit or 0.0))
         self.down = Linear(intermediate_size, hidden_size, precision)
         self._parts: Dict[str, torch.Tensor] = {}
 
