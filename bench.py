@@ -13,6 +13,8 @@ of 6,000 tokens, past the window, at the 27B shape.
 
     python bench.py --telulorn w2048,w4096
         instead of the above: the Telulorn design beside Novotar and Gemma 2 at equal layer sizes, in a line of its own
+    python bench.py --pefitar w2048,w4096
+        instead of the above: the Pefitar design beside Telulorn and Gemma 2 at equal layer sizes, in a line of its own
     python bench.py --novotar w2048,w4096
         instead of the above: prefill and decode throughput of the Novotar design at layer sizes of real models
         (random weights, a few layers), beside Gemma 2 at equal sizes; prints a line of its own
@@ -329,7 +331,25 @@ def telulorn_configs(size, vocab=32768, window=1024):
             "layers": [par, att, par, att], "loop": {"start": 1, "stop": 3, "times": 2}}
 
 
-def novotar_bench(sizes, dtype, steps, warmup, with_telulorn=False):
+def pefitar_configs(size, vocab=32768, window=1024):
+    """A Pefitar configuration of four layers (latent attention, gated attention, latent attention, gated attention), the
+    middle two run twice (six layer runs), at the sizes of novotar_pair_configs: the same width, feed-forward, heads and
+    window.  The latent layers keep 128 plain and 64 rotated dimensions a head, values of 128, a key/value latent of 512
+    and a query latent of three eighths of the width; the gated attention layers see every earlier key."""
+    z = NOVOTAR_SIZES[size]
+    mlp = {"kind": "dense", "ff": z["ff"]}
+    lat = {"type": "latent_attention", "mlp": mlp,
+           "mixer": {"heads": z["heads"], "dim": z["dim"], "rot_dim": 64, "vdim": z["dim"], "q_rank": 3 * z["width"] // 8,
+                     "kv_rank": 512, "scale": (z["dim"] + 64) ** -0.5, "mask": {"size": window},
+                     "rot": {"base": 10000.0, "dims": 64}}}
+    att = {"type": "attention", "mlp": mlp,
+           "mixer": {"heads": z["heads"], "kv_heads": z["kv"], "dim": z["dim"], "vdim": z["dim"], "scale": z["dim"] ** -0.5,
+                     "rot": {"base": 10000.0, "dims": z["dim"] // 2}}}
+    return {"architecture": "Pefitar", "vocab": vocab, "width": z["width"], "norm": {"eps": 1e-6}, "residual_mult": 0.7,
+            "logit_softcap": 30.0, "layers": [lat, att, lat, att], "loop": {"start": 1, "stop": 3, "times": 2}}
+
+
+def novotar_bench(sizes, dtype, steps, warmup, with_telulorn=False, with_pefitar=False):
     out = {}
     for size in sizes:
         if size not in NOVOTAR_SIZES:
@@ -338,6 +358,8 @@ def novotar_bench(sizes, dtype, steps, warmup, with_telulorn=False):
         models = list(zip(("novotar", "gemma2"), novotar_pair_configs(size)))
         if with_telulorn:
             models.insert(0, ("telulorn", telulorn_configs(size)))
+        if with_pefitar:
+            models = [("pefitar", pefitar_configs(size)), ("telulorn", telulorn_configs(size)), models[-1]]
         for name, raw in models:
             run = Run(None, None, dtype, raw=raw)
             r = {"weights_gb": round(run.weight_bytes / 1e9, 3), "layer_runs": len(run.model.lm.plan.schedule)}
@@ -413,6 +435,8 @@ def main() -> int:
                     "sizes instead of the default workload, and print a line of its own")
     ap.add_argument("--telulorn", default="", help="sizes (w2048,w4096): measure the Telulorn design beside Novotar and Gemma 2 at "
                     "equal sizes instead of the default workload, and print a line of its own")
+    ap.add_argument("--pefitar", default="", help="sizes (w2048,w4096): measure the Pefitar design beside Telulorn and Gemma 2 at "
+                    "equal layer sizes, in a line of its own")
     ap.add_argument("--no-peaks", action="store_true", help="skip the measurement of this GPU's own copy and matrix-product rates")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -421,6 +445,13 @@ def main() -> int:
 
     import torch
     torch.cuda.set_device(0)
+    if args.pefitar:
+        steps = min(args.steps, 64)
+        res = novotar_bench([x for x in args.pefitar.split(",") if x], args.dtype, steps, min(args.warmup, 5), with_pefitar=True)
+        print(json.dumps({"metric": "Pefitar beside Telulorn and Gemma 2 at equal layer sizes: prefill and decode, random weights",
+                          "unit": "tokens/s", "n_gpus": 1, "steps": steps, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+                          "data": "synthetic (uniform random token ids, random weights)", "sizes": res}), flush=True)
+        return 0
     if args.telulorn:
         steps = min(args.steps, 64)
         res = novotar_bench([x for x in args.telulorn.split(",") if x], args.dtype, steps, min(args.warmup, 5), with_telulorn=True)
