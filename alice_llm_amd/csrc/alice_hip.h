@@ -180,6 +180,14 @@ int alice_heads_linear(const void* x, int x_dtype, long x_row, int x_head, const
 int alice_latent_attention(const void* q, int dtype, const void* k_pool, void* out, const int* positions,
                            const int* seq_of_token, const int* block_table, int bt_stride, int T, int nH, int kv_rank,
                            int rot_dim, int page_size, float scale, int window, int full_precision, hipStream_t stream);
+// The same on the matrix cores (latent_tiled.hip): bfloat16, kv_rank and rot_dim multiples of 8, together at most 640.
+// The step's tokens are those of n_seqs sequences in order (cu_seqlens).  splits > 1 spreads a row group's key blocks
+// over that many blocks; part then holds splits * T * nH * (kv_rank + 2) floats.
+int alice_latent_tiled_supported(int kv_rank, int rot_dim);
+int alice_latent_tiled_max_splits();
+int alice_latent_tiled(const void* q, const void* pool, void* out, float* part, const int* positions, const int* cu_seqlens,
+                       const int* block_table, int bt_stride, int T, int n_seqs, int nH, int kv_rank, int rot_dim,
+                       int page_size, float scale, int window, int splits, hipStream_t stream);
 int alice_head_gate(void* out, int out_layout, const void* gate, int gate_stride, int T, int nH, int d, hipStream_t stream);
 long alice_attention_decode_workspace(int B, int nH, int d, int splits);
 // out may be absent when splits > 1: the splits are then left in `parts`, [B][nH][splits][ALICE_ATTN_PARTS_HEAD + d]

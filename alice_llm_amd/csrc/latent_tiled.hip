@@ -1,0 +1,342 @@
+// Latent attention on the matrix cores, prompts and single tokens alike.  In the form with the per-head maps on the
+// query's side every head of a token attends over the same cached rows [c (R) | kr (r)], whose first R numbers are
+// the value as well: one "kv head" of D = R + r dimensions for all heads.  So the query rows of a sequence are laid
+// out flat, row = (token - first token) * heads + head, and a block of four waves takes 64 consecutive rows, a wave
+// 16 of them: a staged block of 32 keys serves as many heads of as few tokens as possible (all 16 heads of four
+// tokens with 16 heads; a single token's heads are one wave's rows).
+//
+// A wave computes the transposed score tile S^T = K Q^T with v_mfma_f32_16x16x32_bf16 (keys are the rows, the
+// wave's 16 query rows the columns), so that a lane holds eight scores of ONE query row: maximum and sum are
+// four-lane affairs, and the rounded weights are, as they stand, the second operand of O^T = V^T P^T.  The keys lie
+// in LDS twice, row-major for the first product and transposed (its first DVP dimensions) for the second, in the
+// key order in which the score tiles leave the matrix instruction.  Key blocks that no row of the block sees are
+// not visited.  With splits > 1 (single tokens: few rows, many keys) block z of a row group takes every splits-th
+// run of key blocks and leaves (sum of weighted rows, maximum, sum of weights) for alice_latent_merge.
+// bfloat16 operands, 32-bit scores, softmax and sums.  D and R are multiples of 8, D at most 640.
+#include "common.h"
+#include "alice_hip.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ f32x4 mfma32(u32x4 a, u32x4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+struct LatentArgs {
+  const bf16_t* q;        // [T, nH, D]
+  const bf16_t* pool;     // [pages, 1, page, D]
+  bf16_t* out;            // [T, nH, R]
+  float* part;            // [splits, T nH, R + 2] where splits > 1
+  const int* positions;
+  const int* cu_seqlens;
+  const int* block_table;
+  int bt_stride, n_seqs, nH, R, r, page_size, page_shift;
+  float scale;
+  int window, splits;
+  long rows_total;
+};
+
+constexpr int KT = 32;        // keys a step
+constexpr int VPAD = 40;      // row length of the transposed rows in LDS (32 keys and a pad against bank conflicts)
+constexpr int ROWS = 64;      // query rows a block
+
+template <int DP, int DVP>
+__global__ __launch_bounds__(256) void latent_tiled_kernel(LatentArgs a) {
+  constexpr int KS = DP / 32, ET = DVP / 16;
+  constexpr int KROW = DP + 8;
+  constexpr int NKC = DP / 64, NVC = DVP / 64;          // 16-byte pieces a thread moves a step, for each of the two copies
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  bf16_t (*Ks)[KROW] = reinterpret_cast<bf16_t (*)[KROW]>(lds_raw);                                  // [KT][KROW]
+  bf16_t (*Vt)[VPAD] = reinterpret_cast<bf16_t (*)[VPAD]>(lds_raw + (size_t)KT * KROW * sizeof(bf16_t));   // [DVP][VPAD]
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, g = lane >> 4;
+  const int D = a.R + a.r, R = a.R, nH = a.nH;
+
+  // which 64 rows: the blocks are dealt to the sequences in order, ceil(tokens * heads / 64) each; the last rows of a
+  // sequence have the most keys and go first
+  int idx = gridDim.x - 1 - blockIdx.x, seq = -1, b = 0, n_rows = 0;
+  for (int s = 0; s < a.n_seqs; ++s) {
+    const int sb = a.cu_seqlens[s], se = a.cu_seqlens[s + 1], nt = ((se - sb) * nH + ROWS - 1) / ROWS;
+    if (idx < nt) {
+      seq = s;
+      b = sb;
+      n_rows = (se - sb) * nH;
+      break;
+    }
+    idx -= nt;
+  }
+  if (seq < 0) return;
+  const int rho0 = idx * ROWS, nq = min(ROWS, n_rows - rho0);
+  const int* bt = a.block_table + (size_t)seq * a.bt_stride;
+  const int t_first = b + rho0 / nH, t_last = b + (rho0 + nq - 1) / nH;
+  const int p_first = a.positions[t_first], p_last = p_first + (t_last - t_first);
+  const int rr = wave * 16 + c;
+  const bool valid = rr < nq;
+  const bool wave_on = wave * 16 < nq;
+  const int rho = rho0 + (valid ? rr : 0);
+  const int tq = b + rho / nH;
+  const int qpos = p_first + (tq - t_first);
+  const size_t grow = (size_t)b * nH + rho;              // the row in q and out
+  const int lo_q = a.window > 0 ? qpos + 1 - a.window : 0;
+  const int lo = a.window > 0 ? max(0, p_first + 1 - a.window) : 0;
+  const int t_lo = lo / KT, t_hi = p_last / KT;
+  const int z = blockIdx.y;
+  // this block's steps: z, z + splits, ... of the key blocks t_lo .. t_hi
+  const int n_all = t_hi - t_lo + 1;
+  const int n_steps = n_all > z ? (n_all - z + a.splits - 1) / a.splits : 0;
+
+  u32x4 qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int dim = ks * 32 + g * 8;
+    qf[ks] = u32x4{0u, 0u, 0u, 0u};
+    if (dim < D) qf[ks] = *reinterpret_cast<const u32x4*>(a.q + grow * D + dim);
+  }
+
+  auto row_of = [&](int kp) -> size_t {
+    const int pi = a.page_shift >= 0 ? kp >> a.page_shift : kp / a.page_size;
+    const int sl = a.page_shift >= 0 ? kp & (a.page_size - 1) : kp % a.page_size;
+    return (size_t)bt[pi] * a.page_size + sl;
+  };
+  u32x4 pk[NKC], pv[NVC];
+  auto fetch = [&](int step) {
+    const int key0 = (t_lo + z + step * a.splits) * KT;
+#pragma unroll
+    for (int n = 0; n < NKC; ++n) {
+      const int id = tid + n * 256, key = id / (DP / 8), dim = (id % (DP / 8)) * 8, kp = key0 + key;
+      pk[n] = u32x4{0u, 0u, 0u, 0u};
+      if (key < KT && dim < D && kp <= p_last && kp >= lo) pk[n] = *reinterpret_cast<const u32x4*>(a.pool + row_of(kp) * D + dim);
+    }
+#pragma unroll
+    for (int n = 0; n < NVC; ++n) {
+      const int id = tid + n * 256, key = id % KT, e = (id / KT) * 8, kp = key0 + key;     // neighbouring lanes: neighbouring keys
+      pv[n] = u32x4{0u, 0u, 0u, 0u};
+      if (e < D && kp <= p_last && kp >= lo) pv[n] = *reinterpret_cast<const u32x4*>(a.pool + row_of(kp) * D + e);
+    }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int n = 0; n < NKC; ++n) {
+      const int id = tid + n * 256, key = id / (DP / 8), dim = (id % (DP / 8)) * 8;
+      if (key < KT) *reinterpret_cast<u32x4*>(&Ks[key][dim]) = pk[n];
+    }
+#pragma unroll
+    for (int n = 0; n < NVC; ++n) {
+      const int id = tid + n * 256, key = id % KT, e = (id / KT) * 8;
+      const int col = ((key & 15) >> 2) * 8 + (key & 3) + 4 * (key >> 4);       // the order of the score tiles' rows
+      const uint32_t w[4] = {pv[n][0], pv[n][1], pv[n][2], pv[n][3]};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        Vt[e + 2 * i][col].bits = (uint16_t)(w[i] & 0xffffu);
+        Vt[e + 2 * i + 1][col].bits = (uint16_t)(w[i] >> 16);
+      }
+    }
+  };
+
+  f32x4 oT[ET];
+  float m_run = -INFINITY, l_run = 0.f;
+#pragma unroll
+  for (int et = 0; et < ET; ++et) oT[et] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  if (n_steps > 0) {
+    fetch(0);
+    stage();
+  }
+  __syncthreads();
+  for (int step = 0; step < n_steps; ++step) {
+    const int key0 = (t_lo + z + step * a.splits) * KT;
+    const bool more = step + 1 < n_steps;
+    if (more) fetch(step + 1);
+    if (wave_on) {
+      f32x4 sT[2];
+      sT[0] = sT[1] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) {
+          const u32x4 kf = *reinterpret_cast<const u32x4*>(&Ks[mt * 16 + c][ks * 32 + g * 8]);
+          sT[mt] = mfma32(kf, qf[ks], sT[mt]);
+        }
+      }
+      bool vis[8];
+      bool any = false;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int kp = key0 + (j >> 2) * 16 + g * 4 + (j & 3);
+        vis[j] = valid && kp <= qpos && kp >= lo_q;
+        any = any || vis[j];
+      }
+      if (__ballot(any) != 0ull) {                       // else none of the wave's rows sees a key of this block
+        float sc[8], m_t = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          sc[j] = vis[j] ? sT[j >> 2][j & 3] * a.scale : -INFINITY;
+          m_t = fmaxf(m_t, sc[j]);
+        }
+        m_t = fmaxf(m_t, __shfl_xor(m_t, 16, 64));
+        m_t = fmaxf(m_t, __shfl_xor(m_t, 32, 64));
+        const float m_new = fmaxf(m_run, m_t);
+        float sum = 0.f, corr = 1.f;
+        uint32_t pw[4] = {0u, 0u, 0u, 0u};
+        if (m_new > -INFINITY) {
+          corr = __expf(m_run - m_new);                  // m_run = -inf gives 0
+          float p[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            p[j] = __expf(sc[j] - m_new);
+            sum += p[j];
+          }
+#pragma unroll
+          for (int j = 0; j < 4; ++j) pw[j] = pack_bf16x2(p[2 * j], p[2 * j + 1]);
+          m_run = m_new;
+        }
+        l_run = fmaf(l_run, corr, sum);
+        const u32x4 pf = u32x4{pw[0], pw[1], pw[2], pw[3]};
+#pragma unroll
+        for (int et = 0; et < ET; ++et) {
+          const u32x4 vf = *reinterpret_cast<const u32x4*>(&Vt[et * 16 + c][g * 8]);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) oT[et][i] *= corr;
+          oT[et] = mfma32(vf, pf, oT[et]);
+        }
+      }
+    }
+    __syncthreads();                                     // everybody has read the buffer before it is filled again
+    if (more) stage();
+    __syncthreads();
+  }
+
+  if (!valid) return;
+  float l_tot = l_run;
+  l_tot += __shfl_xor(l_tot, 16, 64);
+  l_tot += __shfl_xor(l_tot, 32, 64);
+  if (a.splits > 1) {
+    float* prow = a.part + ((size_t)z * a.rows_total + grow) * (R + 2);
+#pragma unroll
+    for (int et = 0; et < ET; ++et) {
+      const int e = et * 16 + g * 4;
+      if (e >= R) continue;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) prow[e + i] = oT[et][i];
+    }
+    if (g == 0) {
+      prow[R] = m_run;
+      prow[R + 1] = l_tot;
+    }
+    return;
+  }
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+#pragma unroll
+  for (int et = 0; et < ET; ++et) {
+    const int e = et * 16 + g * 4;
+    if (e >= R) continue;
+    uint2 pkd = {pack_bf16x2(oT[et][0] * inv, oT[et][1] * inv), pack_bf16x2(oT[et][2] * inv, oT[et][3] * inv)};
+    *reinterpret_cast<uint2*>(a.out + grow * R + e) = pkd;
+  }
+}
+
+// One row a block: out = sum_z exp(m_z - M) o_z / sum_z exp(m_z - M) l_z, M the largest of the m_z.
+__global__ __launch_bounds__(128) void latent_merge_kernel(const float* __restrict__ part, bf16_t* __restrict__ out,
+                                                           int splits, long rows_total, int R) {
+  const size_t row = blockIdx.x;
+  float M = -INFINITY;
+  for (int z = 0; z < splits; ++z) M = fmaxf(M, part[((size_t)z * rows_total + row) * (R + 2) + R]);
+  float l = 0.f;
+  for (int z = 0; z < splits; ++z) {
+    const float* p = part + ((size_t)z * rows_total + row) * (R + 2);
+    if (p[R] > -INFINITY) l = fmaf(__expf(p[R] - M), p[R + 1], l);
+  }
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  for (int e = threadIdx.x; e < R; e += blockDim.x) {
+    float o = 0.f;
+    for (int z = 0; z < splits; ++z) {
+      const float* p = part + ((size_t)z * rows_total + row) * (R + 2);
+      if (p[R] > -INFINITY) o = fmaf(__expf(p[R] - M), p[e], o);
+    }
+    out[row * R + e] = f32_to_bf16(o * inv);
+  }
+}
+
+int padded(int n) {
+  const int sizes[] = {64, 128, 192, 256, 384, 512, 576, 640};
+  for (int s : sizes)
+    if (n <= s) return s;
+  return 0;
+}
+
+template <int DP, int DVP>
+int launch(const LatentArgs& a, dim3 grid, hipStream_t stream) {
+  constexpr size_t lds = ((size_t)KT * (DP + 8) + (size_t)DVP * VPAD) * sizeof(bf16_t);
+  static bool raised = false;                            // once a process and instance: more LDS than the static limit
+  if (lds > 48 * 1024 && !raised) {
+    ALICE_CHECK(hipFuncSetAttribute((const void*)latent_tiled_kernel<DP, DVP>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)lds) == hipSuccess, "latent attention: %zu bytes of LDS were refused", lds);
+    raised = true;
+  }
+  latent_tiled_kernel<DP, DVP><<<grid, 256, lds, stream>>>(a);
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int alice_latent_tiled_supported(int kv_rank, int rot_dim) {
+  const int d = kv_rank + rot_dim;
+  return kv_rank >= 8 && kv_rank % 8 == 0 && rot_dim % 8 == 0 && padded(d) != 0;
+}
+
+// The largest number of splits that alice_latent_tiled takes; `part` holds splits * T * nH * (kv_rank + 2) floats.
+extern "C" int alice_latent_tiled_max_splits() { return 32; }
+
+// q: bfloat16 [T, nH (kv_rank + rot_dim)]; pool: bfloat16 [pages, 1, page, kv_rank + rot_dim]; out: bfloat16
+// [T, nH kv_rank].  The step's tokens are those of n_seqs sequences in order (cu_seqlens), each at consecutive
+// positions.  splits > 1 needs `part`.
+extern "C" int alice_latent_tiled(const void* q, const void* pool, void* out, float* part, const int* positions,
+                                  const int* cu_seqlens, const int* block_table, int bt_stride, int T, int n_seqs, int nH,
+                                  int kv_rank, int rot_dim, int page_size, float scale, int window, int splits,
+                                  hipStream_t stream) {
+  ALICE_CHECK(alice_latent_tiled_supported(kv_rank, rot_dim), "latent attention: sizes %d and %d are outside the matrix-core kernel's range (multiples of 8, together at most 640)", kv_rank, rot_dim);
+  ALICE_CHECK(q && pool && out && positions && cu_seqlens && block_table, "latent attention: a pointer is missing");
+  ALICE_CHECK(T >= 0 && n_seqs >= 1 && nH >= 1, "latent attention: bad sizes T=%d n_seqs=%d nH=%d", T, n_seqs, nH);
+  ALICE_CHECK(page_size > 0 && bt_stride > 0 && window >= 0, "latent attention: bad page geometry or window");
+  ALICE_CHECK(splits >= 1 && splits <= alice_latent_tiled_max_splits() && (splits == 1 || part), "latent attention: %d splits, or no room for them", splits);
+  ALICE_CHECK(((uintptr_t)q & 15) == 0 && ((uintptr_t)pool & 15) == 0 && ((uintptr_t)out & 7) == 0, "latent attention: operands are not aligned");
+  if (T == 0) return 0;
+  int page_shift = -1;
+  for (int b = 0; b < 31; ++b)
+    if (page_size == (1 << b)) page_shift = b;
+  const long rows_total = (long)T * nH;
+  LatentArgs a{(const bf16_t*)q, (const bf16_t*)pool, (bf16_t*)out, part, positions, cu_seqlens, block_table, bt_stride, n_seqs,
+               nH, kv_rank, rot_dim, page_size, page_shift, scale, window, splits, rows_total};
+  const int dp = padded(kv_rank + rot_dim);
+  // the second product runs over the row's first DVP dimensions: one size class below the row's where the latent fits
+  dim3 grid(ceil_div(rows_total, ROWS) + n_seqs, splits);
+  int rc = 0;
+#define GO(DP, DVLOW)                                                \
+  case DP:                                                           \
+    rc = (DVLOW < DP && kv_rank <= DVLOW) ? launch<DP, DVLOW>(a, grid, stream) : launch<DP, DP>(a, grid, stream); \
+    break
+  switch (dp) {
+    GO(64, 64);
+    GO(128, 64);
+    GO(192, 128);
+    GO(256, 192);
+    GO(384, 256);
+    GO(512, 384);
+    GO(576, 512);
+    GO(640, 576);
+    default:
+      ALICE_CHECK(false, "latent attention: no kernel for rows of %d", kv_rank + rot_dim);
+  }
+#undef GO
+  if (rc) return rc;
+  ALICE_LAUNCH_CHECK();
+  if (splits > 1) {
+    latent_merge_kernel<<<(unsigned)rows_total, 128, 0, stream>>>(part, (bf16_t*)out, splits, rows_total, kv_rank);
+    ALICE_LAUNCH_CHECK();
+  }
+  return 0;
+}

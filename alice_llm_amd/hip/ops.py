@@ -70,6 +70,9 @@ def _declare(lib) -> None:
         "alice_latent_prepare": [P, I, I, I, I, P, P, F, P, P, P, P, P, I, I, I, P, P, I, I, P],
         "alice_heads_linear": [P, I, L, I, P, I, P, I, L, I, I, I, I, I, I, P, P, P, P],
         "alice_latent_attention": [P, I, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
+        "alice_latent_tiled_supported": [I, I],
+        "alice_latent_tiled_max_splits": [],
+        "alice_latent_tiled": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
         "alice_gla": [P, I, I, I, I, I, P, P, F, F, F, P, I, F, P, I, P, P, P, P, I, I, I, I, I, I, I, P],
         "alice_linear_parts_split": [I, I, I, I, I],
         "alice_linear_parts": [P, I, I, I, P, P, I, I, P],
@@ -847,6 +850,45 @@ def latent_attention(q: torch.Tensor, k_pool: torch.Tensor, out: torch.Tensor, c
     _call("alice_latent_attention", q.data_ptr(), dtype_code(dt), k_pool.data_ptr(), out.data_ptr(), ctx.positions.data_ptr(),
           ctx.seq_of_token.data_ptr(), block_table.data_ptr(), block_table.shape[1], T, num_heads, kv_rank, rot_dim, page_size,
           float(scale), int(window or 0), int(full_precision), _stream())
+
+
+def latent_tiled_supported(dtype: torch.dtype, kv_rank: int, rot_dim: int) -> bool:
+    return dtype == torch.bfloat16 and bool(library().alice_latent_tiled_supported(int(kv_rank), int(rot_dim)))
+
+
+def latent_tiled_splits(n_tokens: int, num_heads: int, max_keys: int) -> int:
+    """Over how many blocks a row group's keys are spread: enough for some 512 blocks in all, every block with at
+    least two runs of 32 keys."""
+    groups = -(-n_tokens * num_heads // 64)
+    key_blocks = -(-max(1, max_keys) // 32) + 1
+    most = min(library().alice_latent_tiled_max_splits(), key_blocks // 2)
+    return max(1, min(most, 512 // max(1, groups)))
+
+
+def latent_attention_tiled(q: torch.Tensor, k_pool: torch.Tensor, out: torch.Tensor, ctx, block_table: torch.Tensor, *,
+                           num_heads: int, kv_rank: int, rot_dim: int, scale: float, window: Optional[int],
+                           splits: int = 1) -> None:
+    """latent_attention on the matrix cores (bfloat16; sizes as latent_tiled_supported says).  The step's tokens are
+    those of ctx.n_seqs sequences in order (ctx.cu_seqlens), each at consecutive positions.  splits > 1 spreads every
+    group of 64 query rows (token, head) over that many blocks along the keys."""
+    T = q.shape[0]
+    _latent_pool(k_pool, kv_rank, rot_dim, torch.bfloat16)
+    _dev(q, "q", torch.bfloat16, (T, num_heads * (kv_rank + rot_dim)))
+    _dev(out, "out", torch.bfloat16, (T, num_heads * kv_rank))
+    _dev(ctx.positions, "positions", torch.int32, (T,))
+    _dev(ctx.cu_seqlens, "cu_seqlens", torch.int32)
+    _dev(block_table, "block_table", torch.int32)
+    page_size = k_pool.shape[2]
+    if ctx.cu_seqlens.numel() < ctx.n_seqs + 1:
+        raise HipLibraryError("cu_seqlens is shorter than the step's sequences")
+    if block_table.dim() != 2 or ctx.max_position // page_size >= block_table.shape[1] or block_table.shape[0] < ctx.n_seqs:
+        raise HipLibraryError(f"position {ctx.max_position} is beyond the block table")
+    part = None
+    if splits > 1:
+        part = torch.empty((splits * T * num_heads * (kv_rank + 2),), dtype=torch.float32, device=q.device)
+    _call("alice_latent_tiled", q.data_ptr(), k_pool.data_ptr(), out.data_ptr(), _opt(part, "part"), ctx.positions.data_ptr(),
+          ctx.cu_seqlens.data_ptr(), block_table.data_ptr(), block_table.shape[1], T, ctx.n_seqs, num_heads, kv_rank, rot_dim,
+          page_size, float(scale), int(window or 0), int(splits), _stream())
 
 
 GLA_MAX_KEY_DIM = 256       # the largest key size the gated linear attention kernel keeps in registers

@@ -129,8 +129,16 @@ class LatentAttention(Part):
         ops.heads_linear(q, self.uk_t, qk, heads=nH, n=R, k=d, rot_dim=r, cos=cos, sin=sin, positions=ctx.positions,
                          max_position=ctx.max_position)
         mixed = torch.empty((T, nH * R), dtype=act, device=dev)
-        ops.latent_attention(qk, cache.k, mixed, ctx, cache.block_table, num_heads=nH, kv_rank=R, rot_dim=r,
-                             scale=self.scale, window=self.window, full_precision=self.precision.full)
+        if not self.precision.full and ops.latent_tiled_supported(act, R, r):
+            # single tokens: few query rows and many keys, so the keys are spread over blocks (the count depends only
+            # on sizes that a captured step holds fixed)
+            most = ctx.max_context if self.window is None else min(ctx.max_context, self.window)
+            splits = ops.latent_tiled_splits(T, nH, most) if ctx.is_decode else 1
+            ops.latent_attention_tiled(qk, cache.k, mixed, ctx, cache.block_table, num_heads=nH, kv_rank=R, rot_dim=r,
+                                       scale=self.scale, window=self.window, splits=splits)
+        else:
+            ops.latent_attention(qk, cache.k, mixed, ctx, cache.block_table, num_heads=nH, kv_rank=R, rot_dim=r,
+                                 scale=self.scale, window=self.window, full_precision=self.precision.full)
         out = torch.empty((T, nH * dv), dtype=act, device=dev)
         ops.heads_linear(mixed, self.uv_t, out, heads=nH, n=dv, k=R)
         return self.o(out, torch.float32, allow_partials=True)
