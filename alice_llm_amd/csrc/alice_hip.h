@@ -188,6 +188,11 @@ int alice_latent_tiled_max_splits();
 int alice_latent_tiled(const void* q, const void* pool, void* out, float* part, const int* positions, const int* cu_seqlens,
                        const int* block_table, int bt_stride, int T, int n_seqs, int nH, int kv_rank, int rot_dim,
                        int page_size, float scale, int window, int splits, hipStream_t stream);
+// A matrix a head on the matrix cores: bfloat16, w as stored [H, n, k]; n a multiple of 4, k and rot_dim of 8.
+int alice_heads_linear_mfma_supported(int n, int k, int rot_dim);
+int alice_heads_linear_mfma(const void* x, long x_row, int x_head, const void* w, void* y, long y_row, int y_head, int T, int H,
+                            int n, int k, int rot_dim, const float* cos_t, const float* sin_t, const int* positions,
+                            hipStream_t stream);
 int alice_head_gate(void* out, int out_layout, const void* gate, int gate_stride, int T, int nH, int d, hipStream_t stream);
 long alice_attention_decode_workspace(int B, int nH, int d, int splits);
 // out may be absent when splits > 1: the splits are then left in `parts`, [B][nH][splits][ALICE_ATTN_PARTS_HEAD + d]

@@ -261,6 +261,99 @@ __global__ __launch_bounds__(128) void latent_merge_kernel(const float* __restri
   }
 }
 
+// ------------------------------------------------------------------------------------- a matrix a head, matrix cores
+// y[t, h, 0:n] = W_h x[t, h, 0:k], W given as stored, [H, n, k] (k contiguous), as the transposed product
+// Y^T = W X^T: the matrix's rows are the first operand's rows, the tokens the columns, so a lane ends with four
+// consecutive outputs of one token.  Both operands come straight from memory in fragment order (16 bytes a lane: eight
+// consecutive k of one row), no LDS and no barrier.  A wave takes MT tiles of 16 tokens and four tiles of 16 outputs;
+// a block's four waves take different tokens (WIDE = false) or different outputs of the same 16 MT tokens (single
+// tokens).  The r numbers behind a head's k inputs are turned in pairs (2i, 2i + 1) by the token's position and put
+// behind its n outputs.
+constexpr int HN = 4;         // output tiles a wave
+
+__device__ __forceinline__ void turn_pair(float u, float v, float cs, float sn, float& a, float& b) {
+  a = fmaf(u, cs, -__fmul_rn(v, sn));
+  b = fmaf(v, cs, __fmul_rn(u, sn));
+}
+
+template <int MT, bool WIDE>
+__global__ __launch_bounds__(256) void heads_linear_mfma_kernel(
+    const bf16_t* __restrict__ x, long x_row, int x_head, const bf16_t* __restrict__ w, bf16_t* __restrict__ y, long y_row,
+    int y_head, int T, int n, int k, int r, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    const int* __restrict__ positions) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, g = lane >> 4;
+  const int h = blockIdx.y;
+  const int block_tokens = 16 * MT * (WIDE ? 1 : 4);
+  const int t0 = blockIdx.x * block_tokens + (WIDE ? 0 : wave * 16 * MT);
+  const int n0 = (blockIdx.z * (WIDE ? 4 : 1) + (WIDE ? wave : 0)) * (16 * HN);
+
+  if (r > 0 && blockIdx.z == 0) {                     // the rotated tail of the block's tokens
+    const int half = r >> 1, tb = blockIdx.x * block_tokens, nt = min(block_tokens, T - tb);
+    for (int i = tid; i < nt * half; i += 256) {
+      const int t = tb + i / half, p = i % half;
+      const bf16_t* src = x + (size_t)t * x_row + (size_t)h * x_head + k;
+      const int pos = positions[t];
+      float y0, y1;
+      turn_pair(bf16_to_f32(src[2 * p]), bf16_to_f32(src[2 * p + 1]), cos_t[(size_t)pos * half + p], sin_t[(size_t)pos * half + p], y0, y1);
+      *reinterpret_cast<uint32_t*>(y + (size_t)t * y_row + (size_t)h * y_head + n + 2 * p) = pack_bf16x2(y0, y1);
+    }
+  }
+  if (t0 >= T || n0 >= n) return;
+
+  f32x4 acc[HN][MT];
+#pragma unroll
+  for (int i = 0; i < HN; ++i)
+#pragma unroll
+    for (int j = 0; j < MT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const bf16_t* wrow[HN];
+  bool w_on[HN];
+#pragma unroll
+  for (int i = 0; i < HN; ++i) {
+    const int row = n0 + i * 16 + c;
+    w_on[i] = row < n;
+    wrow[i] = w + ((size_t)h * n + (w_on[i] ? row : 0)) * k;
+  }
+  const bf16_t* xrow[MT];
+  bool x_on[MT];
+#pragma unroll
+  for (int j = 0; j < MT; ++j) {
+    const int t = t0 + j * 16 + c;
+    x_on[j] = t < T;
+    xrow[j] = x + (size_t)(x_on[j] ? t : 0) * x_row + (size_t)h * x_head;
+  }
+  for (int k0 = 0; k0 < k; k0 += 32) {
+    const int dim = k0 + g * 8;
+    const bool in = dim < k;
+    u32x4 wf[HN], xf[MT];
+#pragma unroll
+    for (int i = 0; i < HN; ++i) {
+      wf[i] = u32x4{0u, 0u, 0u, 0u};
+      if (in && w_on[i]) wf[i] = *reinterpret_cast<const u32x4*>(wrow[i] + dim);
+    }
+#pragma unroll
+    for (int j = 0; j < MT; ++j) {
+      xf[j] = u32x4{0u, 0u, 0u, 0u};
+      if (in && x_on[j]) xf[j] = *reinterpret_cast<const u32x4*>(xrow[j] + dim);
+    }
+#pragma unroll
+    for (int i = 0; i < HN; ++i)
+#pragma unroll
+      for (int j = 0; j < MT; ++j) acc[i][j] = mfma32(wf[i], xf[j], acc[i][j]);
+  }
+#pragma unroll
+  for (int j = 0; j < MT; ++j) {
+    if (!x_on[j]) continue;
+    bf16_t* dst = y + (size_t)(t0 + j * 16 + c) * y_row + (size_t)h * y_head;
+#pragma unroll
+    for (int i = 0; i < HN; ++i) {
+      const int e = n0 + i * 16 + g * 4;
+      if (e >= n) continue;
+      uint2 pkd = {pack_bf16x2(acc[i][j][0], acc[i][j][1]), pack_bf16x2(acc[i][j][2], acc[i][j][3])};
+      *reinterpret_cast<uint2*>(dst + e) = pkd;
+    }
+  }
+}
+
 int padded(int n) {
   const int sizes[] = {64, 128, 192, 256, 384, 512, 576, 640};
   for (int s : sizes)
@@ -338,5 +431,38 @@ extern "C" int alice_latent_tiled(const void* q, const void* pool, void* out, fl
     latent_merge_kernel<<<(unsigned)rows_total, 128, 0, stream>>>(part, (bf16_t*)out, splits, rows_total, kv_rank);
     ALICE_LAUNCH_CHECK();
   }
+  return 0;
+}
+
+extern "C" int alice_heads_linear_mfma_supported(int n, int k, int rot_dim) {
+  return n >= 4 && n % 4 == 0 && k >= 8 && k % 8 == 0 && rot_dim >= 0 && rot_dim % 8 == 0;
+}
+
+// x: bfloat16 rows of x_row elements, head h at h * x_head: [k inputs | rot_dim to be turned]; w: bfloat16 [H, n, k];
+// y: bfloat16 rows of y_row elements, head h at h * y_head: [n outputs | rot_dim turned].
+extern "C" int alice_heads_linear_mfma(const void* x, long x_row, int x_head, const void* w, void* y, long y_row, int y_head,
+                                       int T, int H, int n, int k, int rot_dim, const float* cos_t, const float* sin_t,
+                                       const int* positions, hipStream_t stream) {
+  ALICE_CHECK(alice_heads_linear_mfma_supported(n, k, rot_dim), "heads_linear: sizes n=%d k=%d rot_dim=%d are outside the matrix-core kernel's range", n, k, rot_dim);
+  ALICE_CHECK(x && w && y && T >= 0 && H >= 1 && H <= 65535, "heads_linear: bad sizes T=%d H=%d", T, H);
+  ALICE_CHECK(rot_dim == 0 || (cos_t && sin_t && positions), "heads_linear: a rotated tail needs both tables and the positions");
+  ALICE_CHECK(x_head >= k + rot_dim && y_head >= n + rot_dim && x_row >= (long)(H - 1) * x_head + k + rot_dim &&
+              y_row >= (long)(H - 1) * y_head + n + rot_dim, "heads_linear: the heads do not fit the rows");
+  ALICE_CHECK(x_head % 8 == 0 && x_row % 8 == 0 && y_head % 4 == 0 && y_row % 4 == 0 && ((uintptr_t)x & 15) == 0 &&
+              ((uintptr_t)w & 15) == 0 && ((uintptr_t)y & 7) == 0, "heads_linear: rows or heads are not aligned");
+  if (T == 0) return 0;
+  if (T <= 64) {                                        // few tokens: the waves share them and split the outputs
+    if (T <= 16) {
+      const dim3 grid(1, H, ceil_div(n, 4 * 16 * HN));
+      heads_linear_mfma_kernel<1, true><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)y, y_row, y_head, T, n, k, rot_dim, cos_t, sin_t, positions);
+    } else {
+      const dim3 grid(ceil_div(T, 32), H, ceil_div(n, 4 * 16 * HN));
+      heads_linear_mfma_kernel<2, true><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)y, y_row, y_head, T, n, k, rot_dim, cos_t, sin_t, positions);
+    }
+  } else {
+    const dim3 grid(ceil_div(T, 256), H, ceil_div(n, 16 * HN));
+    heads_linear_mfma_kernel<4, false><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)y, y_row, y_head, T, n, k, rot_dim, cos_t, sin_t, positions);
+  }
+  ALICE_LAUNCH_CHECK();
   return 0;
 }

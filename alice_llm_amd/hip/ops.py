@@ -69,6 +69,8 @@ def _declare(lib) -> None:
         "alice_add_rows": [P, P, P, I, I, P],
         "alice_latent_prepare": [P, I, I, I, I, P, P, F, P, P, P, P, P, I, I, I, P, P, I, I, P],
         "alice_heads_linear": [P, I, L, I, P, I, P, I, L, I, I, I, I, I, I, P, P, P, P],
+        "alice_heads_linear_mfma_supported": [I, I, I],
+        "alice_heads_linear_mfma": [P, L, I, P, P, L, I, I, I, I, I, I, P, P, P, P],
         "alice_latent_attention": [P, I, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
         "alice_latent_tiled_supported": [I, I],
         "alice_latent_tiled_max_splits": [],
@@ -826,6 +828,26 @@ def heads_linear(x: torch.Tensor, wt: torch.Tensor, y: torch.Tensor, *, heads: i
     _call("alice_heads_linear", x.data_ptr(), dtype_code(x.dtype), heads * (k + rot_dim), k + rot_dim, wt.data_ptr(),
           dtype_code(wt.dtype), y.data_ptr(), dtype_code(y.dtype), heads * (n + rot_dim), n + rot_dim, T, heads, n, k,
           rot_dim, c, s_, positions.data_ptr() if rot_dim else None, _stream())
+
+
+def heads_linear_mfma_supported(dtype: torch.dtype, n: int, k: int, rot_dim: int = 0) -> bool:
+    return dtype == torch.bfloat16 and bool(library().alice_heads_linear_mfma_supported(int(n), int(k), int(rot_dim)))
+
+
+def heads_linear_mfma(x: torch.Tensor, w: torch.Tensor, y: torch.Tensor, *, heads: int, n: int, k: int, rot_dim: int = 0,
+                      cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
+                      positions: Optional[torch.Tensor] = None, max_position: int = 0) -> None:
+    """heads_linear on the matrix cores: bfloat16 throughout, and the matrices as stored, w [heads, n, k]."""
+    T = x.shape[0]
+    _dev(x, "x", torch.bfloat16, (T, heads * (k + rot_dim)))
+    _dev(y, "y", torch.bfloat16, (T, heads * (n + rot_dim)))
+    _dev(w, "w", torch.bfloat16, (heads, n, k))
+    c, s_ = _rot_tables(cos, sin, rot_dim, max_position)
+    if rot_dim:
+        _dev(positions, "positions", torch.int32, (T,))
+    _call("alice_heads_linear_mfma", x.data_ptr(), heads * (k + rot_dim), k + rot_dim, w.data_ptr(), y.data_ptr(),
+          heads * (n + rot_dim), n + rot_dim, T, heads, n, k, rot_dim, c, s_, positions.data_ptr() if rot_dim else None,
+          _stream())
 
 
 def latent_attention(q: torch.Tensor, k_pool: torch.Tensor, out: torch.Tensor, ctx, block_table: torch.Tensor, *,

@@ -65,6 +65,7 @@ class LatentAttention(Part):
         self.w_kv_norm: Optional[torch.Tensor] = None
         self.uk_t: Optional[torch.Tensor] = None        # [H, d, R]: head h's map from its plain query to the latent's space
         self.uv_t: Optional[torch.Tensor] = None        # [H, R, dv]: head h's value map, transposed
+        self.uk_mfma = self.uv_mfma = False             # True: kept as [H, outputs, inputs] for the matrix-core kernel
         self._parts: Dict[str, torch.Tensor] = {}
 
     def param_specs(self) -> Dict[str, ParamSpec]:
@@ -106,6 +107,13 @@ class LatentAttention(Part):
         # y[n] = sum_k wt[k, n] x[k]: for the keys' map x is the plain query (k = d, n = R), and Uk_h is [d, R] as stored
         self.uk_t = uk.reshape(self.nH, self.d, self.R).contiguous()
         self.uv_t = uv.reshape(self.nH, self.dv, self.R).transpose(1, 2).contiguous()
+        # the matrix-core kernel reads a head's matrix [outputs, inputs]: only one of the two forms is kept
+        self.uk_mfma = self.uv_mfma = False
+        if not p.full and uk.dtype == torch.bfloat16:
+            if ops.heads_linear_mfma_supported(uk.dtype, self.R, self.d, self.r):
+                self.uk_t, self.uk_mfma = self.uk_t.transpose(1, 2).contiguous(), True
+            if ops.heads_linear_mfma_supported(uv.dtype, self.dv, self.R):
+                self.uv_t, self.uv_mfma = self.uv_t.transpose(1, 2).contiguous(), True
 
     def weight_bytes(self) -> int:
         small = sum(t.numel() * t.element_size() for t in (self.uk_t, self.uv_t))
@@ -126,8 +134,9 @@ class LatentAttention(Part):
                            max_position=ctx.max_position)
         q = self.uq(a, act)                                        # [T, H * (d + r)]
         qk = torch.empty((T, nH * (R + r)), dtype=act, device=dev)
-        ops.heads_linear(q, self.uk_t, qk, heads=nH, n=R, k=d, rot_dim=r, cos=cos, sin=sin, positions=ctx.positions,
-                         max_position=ctx.max_position)
+        (ops.heads_linear_mfma if self.uk_mfma else ops.heads_linear)(
+            q, self.uk_t, qk, heads=nH, n=R, k=d, rot_dim=r, cos=cos, sin=sin, positions=ctx.positions,
+            max_position=ctx.max_position)
         mixed = torch.empty((T, nH * R), dtype=act, device=dev)
         if not self.precision.full and ops.latent_tiled_supported(act, R, r):
             # single tokens: few query rows and many keys, so the keys are spread over blocks (the count depends only
@@ -140,5 +149,5 @@ class LatentAttention(Part):
             ops.latent_attention(qk, cache.k, mixed, ctx, cache.block_table, num_heads=nH, kv_rank=R, rot_dim=r,
                                  scale=self.scale, window=self.window, full_precision=self.precision.full)
         out = torch.empty((T, nH * dv), dtype=act, device=dev)
-        ops.heads_linear(mixed, self.uv_t, out, heads=nH, n=dv, k=R)
+        (ops.heads_linear_mfma if self.uv_mfma else ops.heads_linear)(mixed, self.uv_t, out, heads=nH, n=dv, k=R)
         return self.o(out, torch.float32, allow_partials=True)
