@@ -361,3 +361,136 @@ def telulorn_folder(name: str, seed: int = 0) -> str:
         save_file({k: v.contiguous() for k, v in tensors.items()}, os.path.join(folder, "model.safetensors"))
         _FOLDERS[key] = folder
     return _FOLDERS[key]
+
+
+# --------------------------------------------------------------------------- Pefitar test configurations
+# A: a loop in the middle run twice; the latent layer's sizes all multiples of 8 and all different (query latent 40,
+#    key/value latent 32, plain 16, rotated 8, values 24), a window shorter than a page; grouped kv heads with a part
+#    of the head rotated; one layer without a feed-forward; stream factor 0.7.
+# B: no loop; sizes that fit no tile (width 72, a latent of 44 beside 6 rotated dimensions, heads of 20 / 28); a window
+#    longer than a page; kv heads = heads with the whole head rotated; stream factor 1; no logit cap.
+# C: sizes that suit the matrix cores (latent 128 beside 32 rotated, values 64, heads of 64); a loop over every layer
+#    run three times; a window of exactly a page; one kv head; values wider than keys.
+# D: an attention layer first; a loop over the first layer alone; two latent layers that differ in every size, one
+#    whose window is a single key and one without any window; three query heads a kv head.
+def _pf_lat(heads, dim, rot, vdim, qr, kvr, scale, window, base=1000.0):
+    m = {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": vdim, "q_rank": qr, "kv_rank": kvr, "scale": scale,
+         "rot": {"base": base, "dims": rot}}
+    if window is not None:
+        m["mask"] = {"size": window}
+    return m
+
+
+def _pf_a():
+    lat = _pf_lat(4, 16, 8, 24, 40, 32, 0.3, 9, base=100.0)
+    att = {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 32, "scale": 0.3, "rot": {"base": 100.0, "dims": 8}}
+    mlp = {"kind": "dense", "ff": 96}
+    return {"architecture": "Pefitar", "vocab": 97, "width": 64, "norm": {"eps": 1e-6}, "residual_mult": 0.7, "logit_softcap": 20.0,
+            "layers": [{"type": "latent_attention", "mixer": lat, "mlp": mlp}, {"type": "attention", "mixer": att, "mlp": mlp},
+                       {"type": "latent_attention", "mixer": lat, "mlp": None}],
+            "loop": {"start": 1, "stop": 3, "times": 2}}
+
+
+def _pf_b():
+    lat = _pf_lat(3, 20, 6, 28, 36, 44, 0.25, 70, base=10000.0)
+    att = {"heads": 3, "kv_heads": 3, "dim": 20, "vdim": 20, "scale": 0.3, "rot": {"base": 10000.0, "dims": 20}}
+    mlp = {"kind": "dense", "ff": 100}
+    return {"architecture": "Pefitar", "vocab": 130, "width": 72, "norm": {"eps": 1e-5}, "residual_mult": 1.0,
+            "layers": [{"type": "latent_attention", "mixer": lat, "mlp": mlp}, {"type": "attention", "mixer": att, "mlp": mlp}]}
+
+
+def _pf_c():
+    lat = _pf_lat(4, 32, 32, 64, 64, 128, 0.125, 64, base=500.0)
+    att = {"heads": 4, "kv_heads": 1, "dim": 64, "vdim": 128, "scale": 0.125, "rot": {"base": 500.0, "dims": 32}}
+    mlp = {"kind": "dense", "ff": 256}
+    return {"architecture": "Pefitar", "vocab": 300, "width": 128, "norm": {"eps": 1e-6}, "residual_mult": 0.4, "logit_softcap": 25.0,
+            "layers": [{"type": "attention", "mixer": att, "mlp": mlp}, {"type": "latent_attention", "mixer": lat, "mlp": mlp}],
+            "loop": {"start": 0, "stop": 2, "times": 3}}
+
+
+def _pf_d():
+    att = {"heads": 6, "kv_heads": 2, "dim": 16, "vdim": 24, "scale": 0.25, "rot": {"base": 50.0, "dims": 16}}
+    one = _pf_lat(2, 8, 16, 40, 24, 16, 0.3, 1, base=50.0)
+    free = _pf_lat(5, 24, 8, 8, 16, 56, 0.2, None, base=3000.0)
+    mlp = {"kind": "dense", "ff": 80}
+    return {"architecture": "Pefitar", "vocab": 61, "width": 48, "norm": {"eps": 1e-6}, "residual_mult": 1.3, "logit_softcap": 30.0,
+            "layers": [{"type": "attention", "mixer": att, "mlp": mlp}, {"type": "latent_attention", "mixer": one, "mlp": mlp},
+                       {"type": "latent_attention", "mixer": free, "mlp": None}],
+            "loop": {"start": 0, "stop": 1, "times": 2}}
+
+
+PEFITAR = {"pf-a": _pf_a, "pf-b": _pf_b, "pf-c": _pf_c, "pf-d": _pf_d}
+
+
+def pefitar_tensors(raw: dict, seed: int):
+    """Random tensors for a Pefitar configuration, by name, in bfloat16 on the CPU: matrices N(0, gain^2 / inputs) with
+    gains that make softmaxes sharp and gates open and close; norm weights around 1."""
+    import alice_llm_amd as alice
+    from alice_llm_amd.engine.model import CausalLM
+    from alice_llm_amd.parts import Precision
+    cfg = alice.config_from_dict(raw)
+    specs = CausalLM(cfg.plan(), Precision.of("float32"), "cpu").param_specs()
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, spec in specs.items():
+        shape = tuple(spec.shape)
+        r = torch.randn(shape, generator=g)
+        if len(shape) == 1:
+            t = 1.0 + 0.2 * r
+        elif name == "embed":
+            t = r * 0.5
+        else:
+            gain = 2.5 if name.endswith((".q", ".k", ".g", ".uq", ".uk")) else 1.0
+            t = r * gain / shape[1] ** 0.5
+        out[name] = t.to(torch.bfloat16)
+    return cfg, out
+
+
+class PlainPefitar:
+    """The plain model on given tensors: forward(tokens) -> logits [T, vocab] in 64-bit."""
+
+    def __init__(self, raw, tensors):
+        from plain import pefitar_plain
+        self.P, self.c, self.t = pefitar_plain, raw, {k: v.double() for k, v in tensors.items()}
+
+    @classmethod
+    def from_folder(cls, folder):
+        from plain import pefitar_plain
+        return cls(*pefitar_plain.load_folder(folder))
+
+    def forward(self, tokens, return_layers=False):
+        return self.P.forward(self.c, self.t, tokens, return_stream=return_layers)
+
+    def greedy(self, prompt, n):
+        seq, out = list(prompt), []
+        for _ in range(n):
+            out.append(int(self.forward(seq)[-1].argmax()))
+            seq.append(out[-1])
+        return out
+
+
+def pefitar_pair(name: str, dtype: str, seed: int = 0, device="cuda"):
+    """(the package's model, the plain model) on the same tensors."""
+    raw = PEFITAR[name]()
+    cfg, tensors = pefitar_tensors(raw, seed)
+    model = model_from_tensors(cfg, {k: v.to(device) for k, v in tensors.items()}, dtype)
+    return model, PlainPefitar(raw, tensors)
+
+
+def pefitar_folder(name: str, seed: int = 0) -> str:
+    """A model folder (config.json, model.safetensors in bfloat16) of a Pefitar test configuration."""
+    global _TMP
+    key = ("pefitar", name, seed)
+    if key not in _FOLDERS:
+        from safetensors.torch import save_file
+        if _TMP is None:
+            _TMP = tempfile.TemporaryDirectory(prefix="alice_tests_")
+        folder = os.path.join(_TMP.name, f"{name}-{seed}")
+        os.makedirs(folder, exist_ok=True)
+        raw = PEFITAR[name]()
+        _, tensors = pefitar_tensors(raw, seed)
+        with open(os.path.join(folder, "config.json"), "w") as f:
+            json.dump(raw, f)
+        save_file({k: v.contiguous() for k, v in tensors.items()}, os.path.join(folder, "model.safetensors"))
+        _FOLDERS[key] = folder
+    return _FOLDERS[key]
