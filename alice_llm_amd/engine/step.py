@@ -48,6 +48,11 @@ class StepContext:
     fragment_activations: bool = False
     # every row is wanted, in order (a decode step's "last"): the final norm then needs no gather
     want_every_row: bool = False
+    # the step's sequences and longest context as a captured step of single tokens rounds them, the same in an eager
+    # step of the same tokens: a part that spreads a sequence's keys over blocks chooses how many from these two, so
+    # that both kinds of step add in the same order and give the same bits
+    rounded_seqs: int = 0
+    rounded_context: int = 0
 
 
 Want = Union[str, Sequence[Sequence[int]]]
@@ -128,7 +133,7 @@ class _DecodeGraph:
                                max_new=1, max_context=context, max_position=context - 1, new_lens=[1] * B,
                                captured=True, start_lens=[0] * B, slot_ids=[0] * B,
                                fragment_activations=engine.model.precision.act == torch.bfloat16,
-                               want_every_row=True)
+                               want_every_row=True, rounded_seqs=B, rounded_context=context)
         o = self.offs
         self.shadow[o[2]:o[3]] = np.arange(B)                # constant parts
         self.shadow[o[4]:o[5]] = np.arange(B)
@@ -203,7 +208,7 @@ class _PromptGraph:
                                max_new=T, max_context=context, max_position=context - 1, new_lens=[0] * B,
                                captured=True, start_lens=[0] * B, slot_ids=[0] * B,
                                fragment_activations=engine.model.precision.act == torch.bfloat16,
-                               want_every_row=False)
+                               want_every_row=False, rounded_seqs=B, rounded_context=context)
         self.graph = None
         self.logits = None
 
@@ -394,7 +399,9 @@ class Engine:
                           max_context=max(ctx_lens), max_position=max(ctx_lens) - 1,
                           new_lens=n_new, start_lens=start, slot_ids=list(slots),
                           fragment_activations=self.model.precision.act == torch.bfloat16,
-                          want_every_row=len(rows) == T and (want == "all" or list(rows) == list(range(T))))
+                          want_every_row=len(rows) == T and (want == "all" or list(rows) == list(range(T))),
+                          rounded_seqs=_bucket(B),
+                          rounded_context=min(self.max_positions, -(-max(ctx_lens) // CONTEXT_BUCKET) * CONTEXT_BUCKET))
         logits = self.model.forward(ctx, self.cache, block_tables)
         self.cache.commit(slots, n_new)
         return logits

@@ -139,10 +139,11 @@ class LatentAttention(Part):
             max_position=ctx.max_position)
         mixed = torch.empty((T, nH * R), dtype=act, device=dev)
         if not self.precision.full and ops.latent_tiled_supported(act, R, r):
-            # single tokens: few query rows and many keys, so the keys are spread over blocks (the count depends only
-            # on sizes that a captured step holds fixed)
-            most = ctx.max_context if self.window is None else min(ctx.max_context, self.window)
-            splits = ops.latent_tiled_splits(T, nH, most) if ctx.is_decode else 1
+            # single tokens: few query rows and many keys, so the keys are spread over blocks; how many is chosen from
+            # the step's sizes as a captured step rounds them, so that an eager step of the same tokens adds alike
+            longest = getattr(ctx, "rounded_context", 0) or ctx.max_context
+            most = longest if self.window is None else min(longest, self.window)
+            splits = ops.latent_tiled_splits(getattr(ctx, "rounded_seqs", 0) or T, nH, most) if ctx.is_decode else 1
             ops.latent_attention_tiled(qk, cache.k, mixed, ctx, cache.block_table, num_heads=nH, kv_rank=R, rot_dim=r,
                                        scale=self.scale, window=self.window, splits=splits)
         else:

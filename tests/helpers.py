@@ -440,7 +440,9 @@ def pefitar_tensors(raw: dict, seed: int):
         elif name == "embed":
             t = r * 0.5
         else:
-            gain = 2.5 if name.endswith((".q", ".k", ".g", ".uq", ".uk")) else 1.0
+            # every branch is normed again behind its sublayer, so a rounding inside it reaches the stream undamped:
+            # the gains of the score's two sides are kept lower than the gate's
+            gain = 2.5 if name.endswith(".g") else 1.6 if name.endswith((".q", ".k", ".uq", ".uk")) else 1.0
             t = r * gain / shape[1] ** 0.5
         out[name] = t.to(torch.bfloat16)
     return cfg, out
