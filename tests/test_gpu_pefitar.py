@@ -546,3 +546,70 @@ def test_command_line_generates_from_a_folder():
     for prompt in ([5, 9, 11, 60], [3]):
         ids = plain.greedy(prompt, 5)
         assert ",".join(str(i) for i in ids) in proc.stdout, (ids, proc.stdout[-500:])
+
+
+# ------------------------------------------------------------------ configurations drawn at random
+
+def _drawn_config(seed):
+    """Layers, sizes and constants drawn from a seed: sizes that fit the matrix-core kernels and sizes that fit none,
+    one head and many, every window from a single key to none, loops at the start, the end and over everything."""
+    g = torch.Generator().manual_seed(1000 + seed)
+    pick = lambda xs: xs[int(torch.randint(0, len(xs), (1,), generator=g))]
+    n_layers = pick([1, 2, 3, 4])
+    layers = []
+    for _ in range(n_layers):
+        base = pick([50.0, 1000.0, 20000.0, 500000.0])
+        if pick([0, 1]):
+            heads = pick([1, 2, 3, 4, 6, 8])
+            kv = pick([k for k in (1, 2, 3, 4, 6, 8) if heads % k == 0])
+            dim = pick([8, 12, 16, 24, 32, 40, 64])
+            mixer = {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": pick([8, 12, 20, 32, 48, 64]), "scale": pick([0.1, 0.2, dim ** -0.5]),
+                     "rot": {"base": base, "dims": pick([d for d in (2, 4, 8, 12, 16, 32, 64) if d <= dim])}}
+            if pick([0, 0, 1]):
+                mixer["mask"] = {"size": pick([5, 64, 90])}
+            kind = "attention"
+        else:
+            rot = pick([2, 4, 8, 16, 24, 32])
+            mixer = {"heads": pick([1, 2, 3, 4, 5, 8]), "dim": pick([4, 7, 16, 24, 32, 48]), "rot_dim": rot, "vdim": pick([8, 20, 28, 48, 80]),
+                     "q_rank": pick([16, 30, 64, 96]), "kv_rank": pick([24, 32, 50, 64, 96, 128]), "scale": pick([0.1, 0.15, 0.25]),
+                     "rot": {"base": base, "dims": rot}}
+            w = pick([None, 1, 2, 7, 31, 63, 64, 65, 72, 100, 129])
+            if w is not None:
+                mixer["mask"] = {"size": w}
+            kind = "latent_attention"
+        layers.append({"type": kind, "mixer": mixer, "mlp": None if pick([0, 0, 0, 1]) else {"kind": "dense", "ff": pick([40, 64, 100, 192])}})
+    raw = {"architecture": "Pefitar", "vocab": pick([50, 97, 211, 300]), "width": pick([48, 64, 80, 100, 128]),
+           "norm": {"eps": pick([1e-5, 1e-6])}, "residual_mult": pick([0.3, 0.5, 1.0, 1.4]), "layers": layers}
+    if pick([0, 1]):
+        raw["logit_softcap"] = pick([10.0, 30.0])
+    if pick([0, 1, 1]):
+        a = pick(list(range(n_layers)))
+        raw["loop"] = {"start": a, "stop": pick(list(range(a + 1, n_layers + 1))), "times": pick([1, 2, 3])}
+    return raw
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("seed", range(12))
+def test_drawn_configurations_whole_in_pieces_and_token_by_token(seed, dtype):
+    from helpers import model_from_tensors, pefitar_tensors
+    raw = _drawn_config(seed)
+    cfg, tensors = pefitar_tensors(raw, seed)
+    model = model_from_tensors(cfg, {k: v.to(DEV) for k, v in tensors.items()}, dtype)
+    plain = PlainPefitar(raw, tensors)
+    toks = random_tokens(raw["vocab"], 150, seed)
+    ref = plain.forward(toks)
+    eng = model.engine(max_tokens=512, max_seqs=4)
+    s = eng.open(1)
+    assert_close(eng.step(s, [toks], "all"), ref, dtype, ("whole", raw))
+    eng.close(s)
+    s = eng.open(2)                                             # beside a second request of another length, then token by token
+    other = random_tokens(raw["vocab"], 40, seed + 50)
+    got = [eng.step(s, [toks[:3], other[:9]], "all")[:3], eng.step(s, [toks[3:70], other[9:11]], "all")[:67]]
+    for j in range(70, 150):
+        both = j - 70 < 29                                      # the second request ends after 29 single tokens
+        got.append(eng.step(s if both else s[:1], [[toks[j]], [other[11 + j - 70]]] if both else [[toks[j]]], "last")[:1])
+        if j - 70 == 28:
+            eng.close(s[1:])
+    eng.close(s[:1])
+    assert_close(torch.cat(got), ref, dtype, ("pieces", raw))
+    eng.cache.check_consistent()
