@@ -13,6 +13,14 @@
 // not visited.  With splits > 1 (single tokens: few rows, many keys) block z of a row group takes every splits-th
 // run of key blocks and leaves (sum of weighted rows, maximum, sum of weights) for alice_latent_merge.
 // bfloat16 operands, 32-bit scores, softmax and sums.  D and R are multiples of 8, D at most 640.
+//
+// SINGLE: a step of single tokens with at most 16 heads.  A sequence's rows are then one tile of 16, and the four
+// waves share it instead of three standing by: each takes every fourth 32-dimension slice of the score product (the
+// partial tiles meet in LDS, and every wave does the same softmax on the sum) and every fourth 16-row tile of the
+// transposed output.  A wave's key fragments of its slices come straight from memory in fragment order (16 bytes a
+// lane: eight consecutive dimensions of one key), every element loaded once by one lane, so the row-major copy of the
+// keys in LDS is left out; a wave holds a quarter of the query and of the output.  Several blocks then fit a CU, and
+// one block's walk from page table to rows is covered by the others' arithmetic.
 #include "common.h"
 #include "alice_hip.h"
 
@@ -44,14 +52,17 @@ constexpr int KT = 32;        // keys a step
 constexpr int VPAD = 40;      // row length of the transposed rows in LDS (32 keys and a pad against bank conflicts)
 constexpr int ROWS = 64;      // query rows a block
 
-template <int DP, int DVP>
+template <int DP, int DVP, bool SINGLE>
 __global__ __launch_bounds__(256) void latent_tiled_kernel(LatentArgs a) {
   constexpr int KS = DP / 32, ET = DVP / 16;
+  constexpr int KSW = SINGLE ? (KS + 3) / 4 : KS, ETW = SINGLE ? (ET + 3) / 4 : ET;      // slices and tiles a wave
   constexpr int KROW = DP + 8;
   constexpr int NKC = DP / 64, NVC = DVP / 64;          // 16-byte pieces a thread moves a step, for each of the two copies
   extern __shared__ __align__(16) unsigned char lds_raw[];
+  constexpr size_t KS_BYTES = SINGLE ? 0 : (size_t)KT * KROW * sizeof(bf16_t);                       // SINGLE keeps no row-major copy
   bf16_t (*Ks)[KROW] = reinterpret_cast<bf16_t (*)[KROW]>(lds_raw);                                  // [KT][KROW]
-  bf16_t (*Vt)[VPAD] = reinterpret_cast<bf16_t (*)[VPAD]>(lds_raw + (size_t)KT * KROW * sizeof(bf16_t));   // [DVP][VPAD]
+  bf16_t (*Vt)[VPAD] = reinterpret_cast<bf16_t (*)[VPAD]>(lds_raw + KS_BYTES);                       // [DVP][VPAD]
+  f32x4* Sp = reinterpret_cast<f32x4*>(lds_raw + KS_BYTES + (size_t)DVP * VPAD * sizeof(bf16_t));    // SINGLE: [4][2][64]
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, c = lane & 15, g = lane >> 4;
   const int D = a.R + a.r, R = a.R, nH = a.nH;
@@ -59,24 +70,31 @@ __global__ __launch_bounds__(256) void latent_tiled_kernel(LatentArgs a) {
   // which 64 rows: the blocks are dealt to the sequences in order, ceil(tokens * heads / 64) each; the last rows of a
   // sequence have the most keys and go first
   int idx = gridDim.x - 1 - blockIdx.x, seq = -1, b = 0, n_rows = 0;
-  for (int s = 0; s < a.n_seqs; ++s) {
-    const int sb = a.cu_seqlens[s], se = a.cu_seqlens[s + 1], nt = ((se - sb) * nH + ROWS - 1) / ROWS;
-    if (idx < nt) {
-      seq = s;
-      b = sb;
-      n_rows = (se - sb) * nH;
-      break;
+  if (SINGLE) {                                          // a block a sequence, its one token's heads the rows
+    idx = 0;
+    seq = blockIdx.x;
+    b = a.cu_seqlens[seq];
+    n_rows = nH;
+  } else {
+    for (int s = 0; s < a.n_seqs; ++s) {
+      const int sb = a.cu_seqlens[s], se = a.cu_seqlens[s + 1], nt = ((se - sb) * nH + ROWS - 1) / ROWS;
+      if (idx < nt) {
+        seq = s;
+        b = sb;
+        n_rows = (se - sb) * nH;
+        break;
+      }
+      idx -= nt;
     }
-    idx -= nt;
   }
   if (seq < 0) return;
   const int rho0 = idx * ROWS, nq = min(ROWS, n_rows - rho0);
   const int* bt = a.block_table + (size_t)seq * a.bt_stride;
   const int t_first = b + rho0 / nH, t_last = b + (rho0 + nq - 1) / nH;
   const int p_first = a.positions[t_first], p_last = p_first + (t_last - t_first);
-  const int rr = wave * 16 + c;
+  const int rr = SINGLE ? c : wave * 16 + c;             // SINGLE: every wave has the same 16 rows
   const bool valid = rr < nq;
-  const bool wave_on = wave * 16 < nq;
+  const bool wave_on = SINGLE || wave * 16 < nq;
   const int rho = rho0 + (valid ? rr : 0);
   const int tq = b + rho / nH;
   const int qpos = p_first + (tq - t_first);
@@ -89,12 +107,12 @@ __global__ __launch_bounds__(256) void latent_tiled_kernel(LatentArgs a) {
   const int n_all = t_hi - t_lo + 1;
   const int n_steps = n_all > z ? (n_all - z + a.splits - 1) / a.splits : 0;
 
-  u32x4 qf[KS];
+  u32x4 qf[KSW];                                         // SINGLE: the slices wave, wave + 4, ...
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) {
-    const int dim = ks * 32 + g * 8;
-    qf[ks] = u32x4{0u, 0u, 0u, 0u};
-    if (dim < D) qf[ks] = *reinterpret_cast<const u32x4*>(a.q + grow * D + dim);
+  for (int i = 0; i < KSW; ++i) {
+    const int ks = SINGLE ? wave + 4 * i : i, dim = ks * 32 + g * 8;
+    qf[i] = u32x4{0u, 0u, 0u, 0u};
+    if (ks < KS && dim < D) qf[i] = *reinterpret_cast<const u32x4*>(a.q + grow * D + dim);
   }
 
   auto row_of = [&](int kp) -> size_t {
@@ -102,11 +120,33 @@ __global__ __launch_bounds__(256) void latent_tiled_kernel(LatentArgs a) {
     const int sl = a.page_shift >= 0 ? kp & (a.page_size - 1) : kp % a.page_size;
     return (size_t)bt[pi] * a.page_size + sl;
   };
-  u32x4 pk[NKC], pv[NVC];
-  auto fetch = [&](int step) {
+  // SINGLE: a step's 32 keys lie in one page where pages are a power of two of at least 32 positions, so the page is
+  // looked up once a block and step, by a load that does not depend on the lane, a step ahead of the rows' loads
+  auto page_of = [&](int step) -> int {
+    return SINGLE && a.page_shift >= 5 ? bt[((t_lo + z + step * a.splits) * KT) >> a.page_shift] : -1;
+  };
+  auto row_in = [&](int pg, int kp) -> size_t {
+    return pg >= 0 ? (size_t)pg * a.page_size + (kp & (a.page_size - 1)) : row_of(kp);
+  };
+  u32x4 pk[SINGLE ? 1 : NKC], pv[NVC];
+  u32x4 kfr[SINGLE ? KSW : 1][2];                        // SINGLE: the key fragments of the wave's slices
+  auto fetch_keys = [&](int step, int pg) {              // SINGLE: lane (c, g) takes key c of each tile, dimensions g * 8 ..
     const int key0 = (t_lo + z + step * a.splits) * KT;
 #pragma unroll
-    for (int n = 0; n < NKC; ++n) {
+    for (int i = 0; i < (SINGLE ? KSW : 0); ++i) {
+      const int ks = wave + 4 * i, dim = ks * 32 + g * 8;
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) {
+        const int kp = key0 + mt * 16 + c;
+        kfr[i][mt] = u32x4{0u, 0u, 0u, 0u};
+        if (ks < KS && dim < D && kp <= p_last && kp >= lo) kfr[i][mt] = *reinterpret_cast<const u32x4*>(a.pool + row_in(pg, kp) * D + dim);
+      }
+    }
+  };
+  auto fetch = [&](int step, int pg) {
+    const int key0 = (t_lo + z + step * a.splits) * KT;
+#pragma unroll
+    for (int n = 0; n < (SINGLE ? 0 : NKC); ++n) {
       const int id = tid + n * 256, key = id / (DP / 8), dim = (id % (DP / 8)) * 8, kp = key0 + key;
       pk[n] = u32x4{0u, 0u, 0u, 0u};
       if (key < KT && dim < D && kp <= p_last && kp >= lo) pk[n] = *reinterpret_cast<const u32x4*>(a.pool + row_of(kp) * D + dim);
@@ -115,12 +155,12 @@ __global__ __launch_bounds__(256) void latent_tiled_kernel(LatentArgs a) {
     for (int n = 0; n < NVC; ++n) {
       const int id = tid + n * 256, key = id % KT, e = (id / KT) * 8, kp = key0 + key;     // neighbouring lanes: neighbouring keys
       pv[n] = u32x4{0u, 0u, 0u, 0u};
-      if (e < D && kp <= p_last && kp >= lo) pv[n] = *reinterpret_cast<const u32x4*>(a.pool + row_of(kp) * D + e);
+      if (e < D && kp <= p_last && kp >= lo) pv[n] = *reinterpret_cast<const u32x4*>(a.pool + row_in(pg, kp) * D + e);
     }
   };
   auto stage = [&]() {
 #pragma unroll
-    for (int n = 0; n < NKC; ++n) {
+    for (int n = 0; n < (SINGLE ? 0 : NKC); ++n) {
       const int id = tid + n * 256, key = id / (DP / 8), dim = (id % (DP / 8)) * 8;
       if (key < KT) *reinterpret_cast<u32x4*>(&Ks[key][dim]) = pk[n];
     }
@@ -137,29 +177,50 @@ __global__ __launch_bounds__(256) void latent_tiled_kernel(LatentArgs a) {
     }
   };
 
-  f32x4 oT[ET];
+  f32x4 oT[ETW];                                         // SINGLE: the tiles wave, wave + 4, ...
   float m_run = -INFINITY, l_run = 0.f;
 #pragma unroll
-  for (int et = 0; et < ET; ++et) oT[et] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int et = 0; et < ETW; ++et) oT[et] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  int pg_next = -1;
   if (n_steps > 0) {
-    fetch(0);
+    const int pg = page_of(0);
+    if (n_steps > 1) pg_next = page_of(1);
+    fetch(0, pg);
+    if (SINGLE) fetch_keys(0, pg);
     stage();
   }
   __syncthreads();
   for (int step = 0; step < n_steps; ++step) {
     const int key0 = (t_lo + z + step * a.splits) * KT;
     const bool more = step + 1 < n_steps;
-    if (more) fetch(step + 1);
+    const int pg = pg_next;                              // the next step's page, asked for a step ago
+    if (more) fetch(step + 1, pg);
+    if (step + 2 < n_steps) pg_next = page_of(step + 2);
     if (wave_on) {
       f32x4 sT[2];
       sT[0] = sT[1] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
+      for (int i = 0; i < KSW; ++i) {
+        const int ks = SINGLE ? wave + 4 * i : i;
+        if (ks >= KS) continue;
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt) {
-          const u32x4 kf = *reinterpret_cast<const u32x4*>(&Ks[mt * 16 + c][ks * 32 + g * 8]);
-          sT[mt] = mfma32(kf, qf[ks], sT[mt]);
+          const u32x4 kf = SINGLE ? kfr[SINGLE ? i : 0][mt] : *reinterpret_cast<const u32x4*>(&Ks[mt * 16 + c][ks * 32 + g * 8]);
+          sT[mt] = mfma32(kf, qf[i], sT[mt]);
+        }
+      }
+      if (SINGLE) {                                      // the four waves' partial tiles, summed in one order by all
+        if (more) fetch_keys(step + 1, pg);              // the next step's keys travel during the rest of this one
+        Sp[(wave * 2 + 0) * 64 + lane] = sT[0];
+        Sp[(wave * 2 + 1) * 64 + lane] = sT[1];
+        __syncthreads();
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt) {
+          const f32x4 s0 = Sp[(0 * 2 + mt) * 64 + lane], s1 = Sp[(1 * 2 + mt) * 64 + lane];
+          const f32x4 s2 = Sp[(2 * 2 + mt) * 64 + lane], s3 = Sp[(3 * 2 + mt) * 64 + lane];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) sT[mt][j] = (s0[j] + s1[j]) + (s2[j] + s3[j]);
         }
       }
       bool vis[8];
@@ -197,11 +258,13 @@ __global__ __launch_bounds__(256) void latent_tiled_kernel(LatentArgs a) {
         l_run = fmaf(l_run, corr, sum);
         const u32x4 pf = u32x4{pw[0], pw[1], pw[2], pw[3]};
 #pragma unroll
-        for (int et = 0; et < ET; ++et) {
+        for (int n = 0; n < ETW; ++n) {
+          const int et = SINGLE ? wave + 4 * n : n;
+          if (et >= ET) continue;
           const u32x4 vf = *reinterpret_cast<const u32x4*>(&Vt[et * 16 + c][g * 8]);
 #pragma unroll
-          for (int i = 0; i < 4; ++i) oT[et][i] *= corr;
-          oT[et] = mfma32(vf, pf, oT[et]);
+          for (int i = 0; i < 4; ++i) oT[n][i] *= corr;
+          oT[n] = mfma32(vf, pf, oT[n]);
         }
       }
     }
@@ -217,13 +280,13 @@ __global__ __launch_bounds__(256) void latent_tiled_kernel(LatentArgs a) {
   if (a.splits > 1) {
     float* prow = a.part + ((size_t)z * a.rows_total + grow) * (R + 2);
 #pragma unroll
-    for (int et = 0; et < ET; ++et) {
-      const int e = et * 16 + g * 4;
-      if (e >= R) continue;
+    for (int n = 0; n < ETW; ++n) {
+      const int et = SINGLE ? wave + 4 * n : n, e = et * 16 + g * 4;
+      if (et >= ET || e >= R) continue;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) prow[e + i] = oT[et][i];
+      for (int i = 0; i < 4; ++i) prow[e + i] = oT[n][i];
     }
-    if (g == 0) {
+    if (g == 0 && (!SINGLE || wave == 0)) {
       prow[R] = m_run;
       prow[R + 1] = l_tot;
     }
@@ -231,33 +294,57 @@ __global__ __launch_bounds__(256) void latent_tiled_kernel(LatentArgs a) {
   }
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
 #pragma unroll
-  for (int et = 0; et < ET; ++et) {
-    const int e = et * 16 + g * 4;
-    if (e >= R) continue;
-    uint2 pkd = {pack_bf16x2(oT[et][0] * inv, oT[et][1] * inv), pack_bf16x2(oT[et][2] * inv, oT[et][3] * inv)};
+  for (int n = 0; n < ETW; ++n) {
+    const int et = SINGLE ? wave + 4 * n : n, e = et * 16 + g * 4;
+    if (et >= ET || e >= R) continue;
+    uint2 pkd = {pack_bf16x2(oT[n][0] * inv, oT[n][1] * inv), pack_bf16x2(oT[n][2] * inv, oT[n][3] * inv)};
     *reinterpret_cast<uint2*>(a.out + grow * R + e) = pkd;
   }
 }
 
-// One row a block: out = sum_z exp(m_z - M) o_z / sum_z exp(m_z - M) l_z, M the largest of the m_z.
+// One row a block: out = sum_z exp(m_z - M) o_z / sum_z exp(m_z - M) l_z, M the largest of the m_z.  The splits'
+// maxima and sums are read once into LDS, a split's weight is computed once, and the row's elements are added up with
+// several loads in flight.
 __global__ __launch_bounds__(128) void latent_merge_kernel(const float* __restrict__ part, bf16_t* __restrict__ out,
                                                            int splits, long rows_total, int R) {
   const size_t row = blockIdx.x;
-  float M = -INFINITY;
-  for (int z = 0; z < splits; ++z) M = fmaxf(M, part[((size_t)z * rows_total + row) * (R + 2) + R]);
-  float l = 0.f;
-  for (int z = 0; z < splits; ++z) {
-    const float* p = part + ((size_t)z * rows_total + row) * (R + 2);
-    if (p[R] > -INFINITY) l = fmaf(__expf(p[R] - M), p[R + 1], l);
-  }
-  const float inv = l > 0.f ? 1.f / l : 0.f;
-  for (int e = threadIdx.x; e < R; e += blockDim.x) {
-    float o = 0.f;
-    for (int z = 0; z < splits; ++z) {
-      const float* p = part + ((size_t)z * rows_total + row) * (R + 2);
-      if (p[R] > -INFINITY) o = fmaf(__expf(p[R] - M), p[e], o);
+  const int t = threadIdx.x;
+  __shared__ float mz[32], lz[32], wz[32];
+  if (t < 32) {
+    float m = -INFINITY, l = 0.f;
+    if (t < splits) {
+      const float* p = part + ((size_t)t * rows_total + row) * (R + 2);
+      m = p[R];
+      l = p[R + 1];
     }
-    out[row * R + e] = f32_to_bf16(o * inv);
+    mz[t] = m;
+    lz[t] = l;
+  }
+  __syncthreads();
+  if (t < 32) {
+    float M = -INFINITY, l = 0.f;
+    for (int z = 0; z < splits; ++z) M = fmaxf(M, mz[z]);
+    for (int z = 0; z < splits; ++z)
+      if (mz[z] > -INFINITY) l = fmaf(__expf(mz[z] - M), lz[z], l);
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    wz[t] = mz[t] > -INFINITY ? __expf(mz[t] - M) * inv : 0.f;       // 0 for a split that saw no key
+  }
+  __syncthreads();
+  const size_t stride = (size_t)rows_total * (R + 2);
+  for (int e = t; e < R; e += blockDim.x) {
+    const float* p = part + row * (size_t)(R + 2) + e;
+    float o = 0.f;
+    int z = 0;
+    for (; z + 4 <= splits; z += 4) {                    // four loads in flight
+      const float a0 = p[(size_t)z * stride], a1 = p[(size_t)(z + 1) * stride], a2 = p[(size_t)(z + 2) * stride],
+                  a3 = p[(size_t)(z + 3) * stride];
+      o = fmaf(wz[z], a0, o);
+      o = fmaf(wz[z + 1], a1, o);
+      o = fmaf(wz[z + 2], a2, o);
+      o = fmaf(wz[z + 3], a3, o);
+    }
+    for (; z < splits; ++z) o = fmaf(wz[z], p[(size_t)z * stride], o);
+    out[row * R + e] = f32_to_bf16(o);
   }
 }
 
@@ -361,17 +448,25 @@ int padded(int n) {
   return 0;
 }
 
-template <int DP, int DVP>
-int launch(const LatentArgs& a, dim3 grid, hipStream_t stream) {
-  constexpr size_t lds = ((size_t)KT * (DP + 8) + (size_t)DVP * VPAD) * sizeof(bf16_t);
+template <int DP, int DVP, bool SINGLE>
+int launch_as(const LatentArgs& a, dim3 grid, hipStream_t stream) {
+  constexpr size_t lds = SINGLE ? (size_t)DVP * VPAD * sizeof(bf16_t) + 4 * 2 * 64 * sizeof(f32x4)
+                                : ((size_t)KT * (DP + 8) + (size_t)DVP * VPAD) * sizeof(bf16_t);
   static bool raised = false;                            // once a process and instance: more LDS than the static limit
   if (lds > 48 * 1024 && !raised) {
-    ALICE_CHECK(hipFuncSetAttribute((const void*)latent_tiled_kernel<DP, DVP>, hipFuncAttributeMaxDynamicSharedMemorySize,
+    ALICE_CHECK(hipFuncSetAttribute((const void*)latent_tiled_kernel<DP, DVP, SINGLE>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                     (int)lds) == hipSuccess, "latent attention: %zu bytes of LDS were refused", lds);
     raised = true;
   }
-  latent_tiled_kernel<DP, DVP><<<grid, 256, lds, stream>>>(a);
+  latent_tiled_kernel<DP, DVP, SINGLE><<<grid, 256, lds, stream>>>(a);
   return 0;
+}
+
+// Single tokens of at most 16 heads (every sequence of the step brings one token): a block a sequence and split.
+template <int DP, int DVP>
+int launch(const LatentArgs& a, dim3 grid, bool single, hipStream_t stream) {
+  if (single) return launch_as<DP, DVP, true>(a, dim3(a.n_seqs, grid.y), stream);
+  return launch_as<DP, DVP, false>(a, grid, stream);
 }
 
 }  // namespace
@@ -407,10 +502,11 @@ extern "C" int alice_latent_tiled(const void* q, const void* pool, void* out, fl
   const int dp = padded(kv_rank + rot_dim);
   // the second product runs over the row's first DVP dimensions: one size class below the row's where the latent fits
   dim3 grid(ceil_div(rows_total, ROWS) + n_seqs, splits);
+  const bool single = T == n_seqs && nH <= 16;           // the caller's sequences are in order: one token each
   int rc = 0;
 #define GO(DP, DVLOW)                                                \
   case DP:                                                           \
-    rc = (DVLOW < DP && kv_rank <= DVLOW) ? launch<DP, DVLOW>(a, grid, stream) : launch<DP, DP>(a, grid, stream); \
+    rc = (DVLOW < DP && kv_rank <= DVLOW) ? launch<DP, DVLOW>(a, grid, single, stream) : launch<DP, DP>(a, grid, single, stream); \
     break
   switch (dp) {
     GO(64, 64);
