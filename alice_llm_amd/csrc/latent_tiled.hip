@@ -19,7 +19,8 @@
 // partial tiles meet in LDS, and every wave does the same softmax on the sum) and every fourth 16-row tile of the
 // transposed output.  A wave's key fragments of its slices come straight from memory in fragment order (16 bytes a
 // lane: eight consecutive dimensions of one key), every element loaded once by one lane, so the row-major copy of the
-// keys in LDS is left out; a wave holds a quarter of the query and of the output.  Several blocks then fit a CU, and
+// keys in LDS is left out, and the transposed copy of the next step is written from these same registers: a row is
+// read from memory once.  A wave holds a quarter of the query and of the output.  Several blocks then fit a CU, and
 // one block's walk from page table to rows is covered by the others' arithmetic.
 #include "common.h"
 #include "alice_hip.h"
@@ -128,7 +129,7 @@ __global__ __launch_bounds__(256) void latent_tiled_kernel(LatentArgs a) {
   auto row_in = [&](int pg, int kp) -> size_t {
     return pg >= 0 ? (size_t)pg * a.page_size + (kp & (a.page_size - 1)) : row_of(kp);
   };
-  u32x4 pk[SINGLE ? 1 : NKC], pv[NVC];
+  u32x4 pk[SINGLE ? 1 : NKC], pv[SINGLE ? 1 : NVC];
   u32x4 kfr[SINGLE ? KSW : 1][2];                        // SINGLE: the key fragments of the wave's slices
   auto fetch_keys = [&](int step, int pg) {              // SINGLE: lane (c, g) takes key c of each tile, dimensions g * 8 ..
     const int key0 = (t_lo + z + step * a.splits) * KT;
@@ -152,7 +153,7 @@ __global__ __launch_bounds__(256) void latent_tiled_kernel(LatentArgs a) {
       if (key < KT && dim < D && kp <= p_last && kp >= lo) pk[n] = *reinterpret_cast<const u32x4*>(a.pool + row_of(kp) * D + dim);
     }
 #pragma unroll
-    for (int n = 0; n < NVC; ++n) {
+    for (int n = 0; n < (SINGLE ? 0 : NVC); ++n) {
       const int id = tid + n * 256, key = id % KT, e = (id / KT) * 8, kp = key0 + key;     // neighbouring lanes: neighbouring keys
       pv[n] = u32x4{0u, 0u, 0u, 0u};
       if (e < D && kp <= p_last && kp >= lo) pv[n] = *reinterpret_cast<const u32x4*>(a.pool + row_in(pg, kp) * D + e);
@@ -165,7 +166,22 @@ __global__ __launch_bounds__(256) void latent_tiled_kernel(LatentArgs a) {
       if (key < KT) *reinterpret_cast<u32x4*>(&Ks[key][dim]) = pk[n];
     }
 #pragma unroll
-    for (int n = 0; n < NVC; ++n) {
+    for (int i = 0; i < (SINGLE ? KSW : 0); ++i) {       // SINGLE: the transposed rows from the key fragments
+      const int e = (wave + 4 * i) * 32 + g * 8;
+      if (e >= DVP) continue;
+#pragma unroll
+      for (int mt = 0; mt < 2; ++mt) {
+        const int col = (c >> 2) * 8 + (c & 3) + 4 * mt;
+        const uint32_t w[4] = {kfr[i][mt][0], kfr[i][mt][1], kfr[i][mt][2], kfr[i][mt][3]};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          Vt[e + 2 * j][col].bits = (uint16_t)(w[j] & 0xffffu);
+          Vt[e + 2 * j + 1][col].bits = (uint16_t)(w[j] >> 16);
+        }
+      }
+    }
+#pragma unroll
+    for (int n = 0; n < (SINGLE ? 0 : NVC); ++n) {
       const int id = tid + n * 256, key = id % KT, e = (id / KT) * 8;
       const int col = ((key & 15) >> 2) * 8 + (key & 3) + 4 * (key >> 4);       // the order of the score tiles' rows
       const uint32_t w[4] = {pv[n][0], pv[n][1], pv[n][2], pv[n][3]};

@@ -879,13 +879,13 @@ def latent_tiled_supported(dtype: torch.dtype, kv_rank: int, rot_dim: int) -> bo
 
 
 def latent_tiled_splits(n_tokens: int, num_heads: int, max_keys: int) -> int:
-    """Over how many blocks a row group's keys are spread in a step of single tokens: enough for a block a CU (a
+    """Over how many blocks a row group's keys are spread in a step of single tokens: enough for two blocks a CU (a
     token's heads are a group of their own, 64 rows at most; measured fastest at 1, 8 and 64 tokens of 16 heads over
     1,024 and 8,192 keys), every block with at least two runs of 32 keys."""
     groups = n_tokens * -(-num_heads // 64)
     key_blocks = -(-max(1, max_keys) // 32) + 1
     most = min(library().alice_latent_tiled_max_splits(), key_blocks // 2)
-    return max(1, min(most, 256 // max(1, groups)))
+    return max(1, min(most, 512 // max(1, groups)))
 
 
 def latent_attention_tiled(q: torch.Tensor, k_pool: torch.Tensor, out: torch.Tensor, ctx, block_table: torch.Tensor, *,
