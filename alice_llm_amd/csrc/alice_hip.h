@@ -4,7 +4,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define ALICE_ABI_VERSION 10
+#define ALICE_ABI_VERSION 11
 
 #define ALICE_EPI_NONE 0
 #define ALICE_EPI_GEGLU 1     // W = [gate; up] stacked; epi_param 0: y = gelu_tanh(gate x) * (up x); epi_param = limit > 0:
@@ -182,12 +182,13 @@ int alice_latent_attention(const void* q, int dtype, const void* k_pool, void* o
                            int rot_dim, int page_size, float scale, int window, int full_precision, hipStream_t stream);
 // The same on the matrix cores (latent_tiled.hip): bfloat16, kv_rank and rot_dim multiples of 8, together at most 640.
 // The step's tokens are those of n_seqs sequences in order (cu_seqlens).  splits > 1 spreads a row group's key blocks
-// over that many blocks; part then holds splits * T * nH * (kv_rank + 2) floats.
+// over that many blocks; part then holds splits * T * nH * (kv_rank + 2) floats.  single_tokens: every sequence brings
+// exactly one token (T = n_seqs), which lets the kernel of such steps run where there are at most 16 heads.
 int alice_latent_tiled_supported(int kv_rank, int rot_dim);
 int alice_latent_tiled_max_splits();
 int alice_latent_tiled(const void* q, const void* pool, void* out, float* part, const int* positions, const int* cu_seqlens,
                        const int* block_table, int bt_stride, int T, int n_seqs, int nH, int kv_rank, int rot_dim,
-                       int page_size, float scale, int window, int splits, hipStream_t stream);
+                       int page_size, float scale, int window, int splits, int single_tokens, hipStream_t stream);
 // A matrix a head on the matrix cores: bfloat16, w as stored [H, n, k]; n a multiple of 4, k and rot_dim of 8.
 int alice_heads_linear_mfma_supported(int n, int k, int rot_dim);
 int alice_heads_linear_mfma(const void* x, long x_row, int x_head, const void* w, void* y, long y_row, int y_head, int T, int H,

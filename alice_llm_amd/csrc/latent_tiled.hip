@@ -497,11 +497,11 @@ extern "C" int alice_latent_tiled_max_splits() { return 32; }
 
 // q: bfloat16 [T, nH (kv_rank + rot_dim)]; pool: bfloat16 [pages, 1, page, kv_rank + rot_dim]; out: bfloat16
 // [T, nH kv_rank].  The step's tokens are those of n_seqs sequences in order (cu_seqlens), each at consecutive
-// positions.  splits > 1 needs `part`.
+// positions.  splits > 1 needs `part`.  single_tokens: the caller's word that every sequence brings one token.
 extern "C" int alice_latent_tiled(const void* q, const void* pool, void* out, float* part, const int* positions,
                                   const int* cu_seqlens, const int* block_table, int bt_stride, int T, int n_seqs, int nH,
                                   int kv_rank, int rot_dim, int page_size, float scale, int window, int splits,
-                                  hipStream_t stream) {
+                                  int single_tokens, hipStream_t stream) {
   ALICE_CHECK(alice_latent_tiled_supported(kv_rank, rot_dim), "latent attention: sizes %d and %d are outside the matrix-core kernel's range (multiples of 8, together at most 640)", kv_rank, rot_dim);
   ALICE_CHECK(q && pool && out && positions && cu_seqlens && block_table, "latent attention: a pointer is missing");
   ALICE_CHECK(T >= 0 && n_seqs >= 1 && nH >= 1, "latent attention: bad sizes T=%d n_seqs=%d nH=%d", T, n_seqs, nH);
@@ -518,7 +518,8 @@ extern "C" int alice_latent_tiled(const void* q, const void* pool, void* out, fl
   const int dp = padded(kv_rank + rot_dim);
   // the second product runs over the row's first DVP dimensions: one size class below the row's where the latent fits
   dim3 grid(ceil_div(rows_total, ROWS) + n_seqs, splits);
-  const bool single = T == n_seqs && nH <= 16;           // the caller's sequences are in order: one token each
+  ALICE_CHECK(!single_tokens || T == n_seqs, "latent attention: a step of single tokens has %d tokens for %d sequences", T, n_seqs);
+  const bool single = single_tokens && nH <= 16;
   int rc = 0;
 #define GO(DP, DVLOW)                                                \
   case DP:                                                           \

@@ -18,7 +18,7 @@ from ..csrc import build as _build
 EPI_NONE, EPI_GEGLU, EPI_SOFTCAP = 0, 1, 2
 LAYOUT_ROW, LAYOUT_FRAG16 = 0, 1
 LINEAR_AUTO, LINEAR_GENERIC, LINEAR_SKINNY, LINEAR_MFMA, LINEAR_TILED_W16, LINEAR_TILED_W32 = 0, 1, 2, 3, 4, 5
-ABI_VERSION = 10
+ABI_VERSION = 11
 GATED_SILU = -1.0        # epi_param of EPI_GEGLU that picks silu(gate) * up
 UNARY_RELU2 = -1.0       # epi_param of EPI_SOFTCAP that picks the square of max(y, 0) instead of the capped form
 
@@ -74,7 +74,7 @@ def _declare(lib) -> None:
         "alice_latent_attention": [P, I, P, P, P, P, P, I, I, I, I, I, I, F, I, I, P],
         "alice_latent_tiled_supported": [I, I],
         "alice_latent_tiled_max_splits": [],
-        "alice_latent_tiled": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P],
+        "alice_latent_tiled": [P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, I, P],
         "alice_gla": [P, I, I, I, I, I, P, P, F, F, F, P, I, F, P, I, P, P, P, P, I, I, I, I, I, I, I, P],
         "alice_linear_parts_split": [I, I, I, I, I],
         "alice_linear_parts": [P, I, I, I, P, P, I, I, P],
@@ -890,10 +890,11 @@ def latent_tiled_splits(n_tokens: int, num_heads: int, max_keys: int) -> int:
 
 def latent_attention_tiled(q: torch.Tensor, k_pool: torch.Tensor, out: torch.Tensor, ctx, block_table: torch.Tensor, *,
                            num_heads: int, kv_rank: int, rot_dim: int, scale: float, window: Optional[int],
-                           splits: int = 1) -> None:
+                           splits: int = 1, single_tokens: bool = False) -> None:
     """latent_attention on the matrix cores (bfloat16; sizes as latent_tiled_supported says).  The step's tokens are
     those of ctx.n_seqs sequences in order (ctx.cu_seqlens), each at consecutive positions.  splits > 1 spreads every
-    group of 64 query rows (token, head) over that many blocks along the keys."""
+    group of 64 query rows (token, head) over that many blocks along the keys.  single_tokens: every sequence of the
+    step brings exactly one token (a decode step); with at most 16 heads the kernel of such steps then runs."""
     T = q.shape[0]
     _latent_pool(k_pool, kv_rank, rot_dim, torch.bfloat16)
     _dev(q, "q", torch.bfloat16, (T, num_heads * (kv_rank + rot_dim)))
@@ -904,6 +905,8 @@ def latent_attention_tiled(q: torch.Tensor, k_pool: torch.Tensor, out: torch.Ten
     page_size = k_pool.shape[2]
     if ctx.cu_seqlens.numel() < ctx.n_seqs + 1:
         raise HipLibraryError("cu_seqlens is shorter than the step's sequences")
+    if single_tokens and T != ctx.n_seqs:
+        raise HipLibraryError(f"a step of single tokens has {T} tokens for {ctx.n_seqs} sequences")
     if block_table.dim() != 2 or ctx.max_position // page_size >= block_table.shape[1] or block_table.shape[0] < ctx.n_seqs:
         raise HipLibraryError(f"position {ctx.max_position} is beyond the block table")
     part = None
@@ -911,7 +914,7 @@ def latent_attention_tiled(q: torch.Tensor, k_pool: torch.Tensor, out: torch.Ten
         part = torch.empty((splits * T * num_heads * (kv_rank + 2),), dtype=torch.float32, device=q.device)
     _call("alice_latent_tiled", q.data_ptr(), k_pool.data_ptr(), out.data_ptr(), _opt(part, "part"), ctx.positions.data_ptr(),
           ctx.cu_seqlens.data_ptr(), block_table.data_ptr(), block_table.shape[1], T, ctx.n_seqs, num_heads, kv_rank, rot_dim,
-          page_size, float(scale), int(window or 0), int(splits), _stream())
+          page_size, float(scale), int(window or 0), int(splits), int(bool(single_tokens)), _stream())
 
 
 GLA_MAX_KEY_DIM = 256       # the largest key size the gated linear attention kernel keeps in registers

@@ -145,7 +145,7 @@ class LatentAttention(Part):
             most = longest if self.window is None else min(longest, self.window)
             splits = ops.latent_tiled_splits(getattr(ctx, "rounded_seqs", 0) or T, nH, most) if ctx.is_decode else 1
             ops.latent_attention_tiled(qk, cache.k, mixed, ctx, cache.block_table, num_heads=nH, kv_rank=R, rot_dim=r,
-                                       scale=self.scale, window=self.window, splits=splits)
+                                       scale=self.scale, window=self.window, splits=splits, single_tokens=ctx.is_decode)
         else:
             ops.latent_attention(qk, cache.k, mixed, ctx, cache.block_table, num_heads=nH, kv_rank=R, rot_dim=r,
                                  scale=self.scale, window=self.window, full_precision=self.precision.full)

@@ -241,11 +241,15 @@ def test_attention_over_latent_rows_at_the_windows_edges_and_far_back(dtype, H, 
     assert max_err(out.view(-1, H, R), ref[singles]) < tol, singles
     if tiled:
         most = T if window is None else min(T, window)
-        for splits in sorted({1, 2, ops.latent_tiled_splits(len(singles), H, most)}):
+        # by the kernel of single tokens (the waves share a token's heads) and by the prompt kernel's mapping
+        for splits, single in [(s_, w_) for s_ in sorted({1, 2, ops.latent_tiled_splits(len(singles), H, most)}) for w_ in (True, False)]:
             out2 = torch.full_like(out, 9.0)
             ops.latent_attention_tiled(qs, pool, out2, ctx, bt, num_heads=H, kv_rank=R, rot_dim=r, scale=scale, window=window,
-                                       splits=splits)
-            assert max_err(out2.view(-1, H, R), ref[singles]) < tol, ("tiled", splits)
+                                       splits=splits, single_tokens=single)
+            assert max_err(out2.view(-1, H, R), ref[singles]) < tol, ("tiled", splits, single)
+        with pytest.raises(ops.HipLibraryError, match="single tokens"):         # two tokens of one sequence are no such step
+            ops.latent_attention_tiled(qs[:2].contiguous(), pool, out[:2], _latent_ctx([2], [0]), bt, num_heads=H, kv_rank=R,
+                                       rot_dim=r, scale=scale, window=window, single_tokens=True)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
