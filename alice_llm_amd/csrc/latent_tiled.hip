@@ -121,10 +121,10 @@ __global__ __launch_bounds__(256) void latent_tiled_kernel(LatentArgs a) {
     const int sl = a.page_shift >= 0 ? kp & (a.page_size - 1) : kp % a.page_size;
     return (size_t)bt[pi] * a.page_size + sl;
   };
-  // SINGLE: a step's 32 keys lie in one page where pages are a power of two of at least 32 positions, so the page is
-  // looked up once a block and step, by a load that does not depend on the lane, a step ahead of the rows' loads
+  // A step's 32 keys lie in one page where pages are a power of two of at least 32 positions, so the page is looked
+  // up once a block and step, by a load that does not depend on the lane, a step ahead of the rows' loads
   auto page_of = [&](int step) -> int {
-    return SINGLE && a.page_shift >= 5 ? bt[((t_lo + z + step * a.splits) * KT) >> a.page_shift] : -1;
+    return a.page_shift >= 5 ? bt[((t_lo + z + step * a.splits) * KT) >> a.page_shift] : -1;
   };
   auto row_in = [&](int pg, int kp) -> size_t {
     return pg >= 0 ? (size_t)pg * a.page_size + (kp & (a.page_size - 1)) : row_of(kp);
