@@ -253,7 +253,7 @@ def test_attention_over_latent_rows_at_the_windows_edges_and_far_back(dtype, H, 
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,G,d,dv,T", [(6, 1, 64, 48, 700), (4, 2, 16, 32, 330), (3, 3, 20, 20, 200), (6, 2, 16, 24, 130)])
+@pytest.mark.parametrize("H,G,d,dv,T", [(8, 1, 64, 32, 700), (4, 2, 16, 32, 330), (3, 3, 20, 20, 200), (6, 2, 16, 24, 130)])
 def test_gated_attention_finds_a_key_hundreds_of_tokens_back(dtype, H, G, d, dv, T):
     """Every earlier key is visible: a marker key at position 3 carries the last rows over hundreds of others; the
     elementwise gate (rows of a wider matrix) closes some output elements and opens others."""
@@ -562,7 +562,7 @@ def _drawn_config(seed):
     n_layers = pick([1, 2, 3, 4])
     layers = []
     for _ in range(n_layers):
-        base = pick([50.0, 1000.0, 20000.0, 500000.0])
+        base = pick([50.0, 1000.0, 30000.0, 500000.0])
         if pick([0, 1]):
             heads = pick([1, 2, 3, 4, 6, 8])
             kv = pick([k for k in (1, 2, 3, 4, 6, 8) if heads % k == 0])
@@ -577,7 +577,7 @@ def _drawn_config(seed):
             mixer = {"heads": pick([1, 2, 3, 4, 5, 8]), "dim": pick([4, 7, 16, 24, 32, 48]), "rot_dim": rot, "vdim": pick([8, 20, 28, 48, 80]),
                      "q_rank": pick([16, 30, 64, 96]), "kv_rank": pick([24, 32, 50, 64, 96, 128]), "scale": pick([0.1, 0.15, 0.25]),
                      "rot": {"base": base, "dims": rot}}
-            w = pick([None, 1, 2, 7, 31, 63, 64, 65, 72, 100, 129])
+            w = pick([None, 1, 2, 7, 31, 63, 64, 65, 70, 100, 129])
             if w is not None:
                 mixer["mask"] = {"size": w}
             kind = "latent_attention"
