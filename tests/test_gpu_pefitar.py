@@ -322,6 +322,35 @@ def test_silu_gated_feed_forward(dtype, T, W, I):
     assert max_err(out, ref) < (2e-5 if dtype == "float32" else 3e-2) * max(1.0, float(ref.abs().max()))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,W,mult", [(1, 64, 0.7), (9, 72, 1.0), (70, 100, 1.3), (300, 128, 0.4), (5, 2048, 0.25)])
+def test_norms_around_a_sublayer_with_the_streams_factor(dtype, T, W, mult):
+    """x + m N_b(branch) and then N_a of the sum, by the fused add-and-norm kernel and by the add alone: eps inside the
+    root (a branch row of tiny numbers), weights stored in bfloat16 and kept in 32-bit with the factor folded in, the
+    stream in 32-bit whatever the arithmetic."""
+    from alice_llm_amd.parts import NORMS
+    from alice_llm_amd.parts.stream import ResidualStream
+    prec, eps = Precision.of(dtype), 1e-5
+    behind = NORMS.get("rmsnorm")(prec, dim=W, eps=eps, tensor_name="", output_scale=mult, keep_float32=True)
+    ahead = NORMS.get("rmsnorm")(prec, dim=W, eps=eps, tensor_name="", keep_float32=True)
+    wb, wa = (1.0 + 0.3 * rnd(W, seed=1)).to(torch.bfloat16), (1.0 + 0.3 * rnd(W, seed=2)).to(torch.bfloat16)
+    behind.assign("", wb.to(DEV))
+    ahead.assign("", wa.to(DEV))
+    assert behind.weight.dtype == torch.float32 and ahead.weight.dtype == torch.float32
+    x, branch = rnd(T, W, seed=3, scale=2.0), rnd(T, W, seed=4, scale=5.0)
+    branch[0] *= 1e-4
+    want_x = x.double() + mult * P.rms_norm(branch.double(), wb.double(), eps)
+    want_h = P.rms_norm(want_x, wa.double(), eps)
+    for fused in (True, False):
+        stream = ResidualStream(x.clone().to(DEV), prec)
+        stream.push(branch.to(DEV), behind)
+        if fused:
+            h = stream.normed(ahead)
+            assert max_err(h, want_h) < (3e-6 if dtype == "float32" else 2e-2) * 4
+        stream.flush()
+        assert stream.x.dtype == torch.float32 and max_err(stream.x, want_x) < 2e-5
+
+
 # ------------------------------------------------------------------ the model through the engine
 
 @pytest.mark.parametrize("name,dtype", CASES)
