@@ -370,16 +370,16 @@ __global__ __launch_bounds__(128) void latent_merge_kernel(const float* __restri
 // consecutive outputs of one token.  Both operands come straight from memory in fragment order (16 bytes a lane: eight
 // consecutive k of one row), no LDS and no barrier.  A wave takes MT tiles of 16 tokens and four tiles of 16 outputs;
 // a block's four waves take different tokens (WIDE = false) or different outputs of the same 16 MT tokens (single
-// tokens).  The r numbers behind a head's k inputs are turned in pairs (2i, 2i + 1) by the token's position and put
+// tokens, a tile of 16 outputs a wave: the matrices are all there is to read, so the more blocks read them the better).  The r numbers behind a head's k inputs are turned in pairs (2i, 2i + 1) by the token's position and put
 // behind its n outputs.
-constexpr int HN = 4;         // output tiles a wave
+constexpr int HN = 4;         // output tiles a wave where the waves take different tokens
 
 __device__ __forceinline__ void turn_pair(float u, float v, float cs, float sn, float& a, float& b) {
   a = fmaf(u, cs, -__fmul_rn(v, sn));
   b = fmaf(v, cs, __fmul_rn(u, sn));
 }
 
-template <int MT, bool WIDE>
+template <int MT, bool WIDE, int HT>
 __global__ __launch_bounds__(256) void heads_linear_mfma_kernel(
     const bf16_t* __restrict__ x, long x_row, int x_head, const bf16_t* __restrict__ w, bf16_t* __restrict__ y, long y_row,
     int y_head, int T, int n, int k, int r, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
@@ -388,7 +388,7 @@ __global__ __launch_bounds__(256) void heads_linear_mfma_kernel(
   const int h = blockIdx.y;
   const int block_tokens = 16 * MT * (WIDE ? 1 : 4);
   const int t0 = blockIdx.x * block_tokens + (WIDE ? 0 : wave * 16 * MT);
-  const int n0 = (blockIdx.z * (WIDE ? 4 : 1) + (WIDE ? wave : 0)) * (16 * HN);
+  const int n0 = (blockIdx.z * (WIDE ? 4 : 1) + (WIDE ? wave : 0)) * (16 * HT);
 
   if (r > 0 && blockIdx.z == 0) {                     // the rotated tail of the block's tokens
     const int half = r >> 1, tb = blockIdx.x * block_tokens, nt = min(block_tokens, T - tb);
@@ -403,15 +403,15 @@ __global__ __launch_bounds__(256) void heads_linear_mfma_kernel(
   }
   if (t0 >= T || n0 >= n) return;
 
-  f32x4 acc[HN][MT];
+  f32x4 acc[HT][MT];
 #pragma unroll
-  for (int i = 0; i < HN; ++i)
+  for (int i = 0; i < HT; ++i)
 #pragma unroll
     for (int j = 0; j < MT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const bf16_t* wrow[HN];
-  bool w_on[HN];
+  const bf16_t* wrow[HT];
+  bool w_on[HT];
 #pragma unroll
-  for (int i = 0; i < HN; ++i) {
+  for (int i = 0; i < HT; ++i) {
     const int row = n0 + i * 16 + c;
     w_on[i] = row < n;
     wrow[i] = w + ((size_t)h * n + (w_on[i] ? row : 0)) * k;
@@ -427,9 +427,9 @@ __global__ __launch_bounds__(256) void heads_linear_mfma_kernel(
   for (int k0 = 0; k0 < k; k0 += 32) {
     const int dim = k0 + g * 8;
     const bool in = dim < k;
-    u32x4 wf[HN], xf[MT];
+    u32x4 wf[HT], xf[MT];
 #pragma unroll
-    for (int i = 0; i < HN; ++i) {
+    for (int i = 0; i < HT; ++i) {
       wf[i] = u32x4{0u, 0u, 0u, 0u};
       if (in && w_on[i]) wf[i] = *reinterpret_cast<const u32x4*>(wrow[i] + dim);
     }
@@ -439,7 +439,7 @@ __global__ __launch_bounds__(256) void heads_linear_mfma_kernel(
       if (in && x_on[j]) xf[j] = *reinterpret_cast<const u32x4*>(xrow[j] + dim);
     }
 #pragma unroll
-    for (int i = 0; i < HN; ++i)
+    for (int i = 0; i < HT; ++i)
 #pragma unroll
       for (int j = 0; j < MT; ++j) acc[i][j] = mfma32(wf[i], xf[j], acc[i][j]);
   }
@@ -448,7 +448,7 @@ __global__ __launch_bounds__(256) void heads_linear_mfma_kernel(
     if (!x_on[j]) continue;
     bf16_t* dst = y + (size_t)(t0 + j * 16 + c) * y_row + (size_t)h * y_head;
 #pragma unroll
-    for (int i = 0; i < HN; ++i) {
+    for (int i = 0; i < HT; ++i) {
       const int e = n0 + i * 16 + g * 4;
       if (e >= n) continue;
       uint2 pkd = {pack_bf16x2(acc[i][j][0], acc[i][j][1]), pack_bf16x2(acc[i][j][2], acc[i][j][3])};
@@ -566,15 +566,15 @@ extern "C" int alice_heads_linear_mfma(const void* x, long x_row, int x_head, co
   if (T == 0) return 0;
   if (T <= 64) {                                        // few tokens: the waves share them and split the outputs
     if (T <= 16) {
-      const dim3 grid(1, H, ceil_div(n, 4 * 16 * HN));
-      heads_linear_mfma_kernel<1, true><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)y, y_row, y_head, T, n, k, rot_dim, cos_t, sin_t, positions);
+      const dim3 grid(1, H, ceil_div(n, 4 * 16));
+      heads_linear_mfma_kernel<1, true, 1><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)y, y_row, y_head, T, n, k, rot_dim, cos_t, sin_t, positions);
     } else {
-      const dim3 grid(ceil_div(T, 32), H, ceil_div(n, 4 * 16 * HN));
-      heads_linear_mfma_kernel<2, true><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)y, y_row, y_head, T, n, k, rot_dim, cos_t, sin_t, positions);
+      const dim3 grid(ceil_div(T, 32), H, ceil_div(n, 4 * 16));
+      heads_linear_mfma_kernel<2, true, 1><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)y, y_row, y_head, T, n, k, rot_dim, cos_t, sin_t, positions);
     }
   } else {
     const dim3 grid(ceil_div(T, 256), H, ceil_div(n, 16 * HN));
-    heads_linear_mfma_kernel<4, false><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)y, y_row, y_head, T, n, k, rot_dim, cos_t, sin_t, positions);
+    heads_linear_mfma_kernel<4, false, HN><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)y, y_row, y_head, T, n, k, rot_dim, cos_t, sin_t, positions);
   }
   ALICE_LAUNCH_CHECK();
   return 0;
