@@ -5,9 +5,11 @@ from .gemma2 import Gemma2Config
 from .novotar import NovotarConfig
 from .telulorn import TelulornConfig
 from .pefitar import PefitarConfig
+from .vifirax import VifiraxConfig
 from . import presets
 
 register_architecture("Gemma2ForCausalLM", Gemma2Config, model_type="gemma2")
 register_architecture("Novotar", NovotarConfig)
 register_architecture("Telulorn", TelulornConfig)
 register_architecture("Pefitar", PefitarConfig)
+register_architecture("Vifirax", VifiraxConfig)

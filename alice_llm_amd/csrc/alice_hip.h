@@ -4,7 +4,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
-#define ALICE_ABI_VERSION 11
+#define ALICE_ABI_VERSION 12
 
 #define ALICE_EPI_NONE 0
 #define ALICE_EPI_GEGLU 1     // W = [gate; up] stacked; epi_param 0: y = gelu_tanh(gate x) * (up x); epi_param = limit > 0:
@@ -156,7 +156,10 @@ int alice_qkv_prepare(const void* rows, int rows_dtype, int row_width, const flo
                       void* v_pool, int out_dtype, const float* cos_t, const float* sin_t, int rotary_dim,
                       int interleaved, const float* vcos, const float* vsin, const int* positions,
                       const int* seq_of_token, const int* block_table, int bt_stride, int T, int nH, int nKV,
-                      int d, int dv, int page_size, int n_pages, hipStream_t stream);
+                      int d, int dv, int page_size, int n_pages, const float* norm_w, float norm_eps, float* inv_rms,
+                      hipStream_t stream);
+// (norm_w: float32 [nH d + nKV d] or null: the q columns and the k columns are each RMS-normed over the whole
+// projection, after the bias and before the rotation; inv_rms: float32 [T, 2] workspace.)
 // x[t, c] += a[t, c] + v[c] (either may be null)
 int alice_add_rows(float* x, const float* a, const float* v, int T, int W, hipStream_t stream);
 // Gated linear attention over a step's tokens, see gla.hip.
@@ -164,6 +167,33 @@ int alice_gla(const float* rows, int row_w, int q_col, int k_col, int v_col, int
               const float* z_bias, float tau, float q_scale, float out_scale, const void* norm_w, int w_dtype, float eps, void* out,
               int out_dtype, float* work, const int* cu_seqlens, const int* slots, float* S, int T, int n_seqs,
               int n_slots, int H, int d, int dv, int columns, hipStream_t stream);
+// Short causal convolution per channel over each sequence's tokens, with the last taps - 1 inputs of earlier steps in
+// state [slots, channels, taps - 1]; act 1: silu.  See recurrent.hip for this and the four entries below.
+int alice_short_conv(const float* rows, int row_w, int col0, int channels, int taps, const float* w, const float* bias,
+                     float* state, float* out, int act, const int* cu_seqlens, const int* seq_of_token, const int* slots,
+                     int T, int n_seqs, hipStream_t stream);
+// step = softplus(rows[:, dt_col + h] + dt_bias[h]), decay = exp(-exp(a_log[h]) step), both [T, H]
+int alice_ssm_prepare(const float* rows, int row_w, int dt_col, const float* dt_bias, const float* a_log, float* step,
+                      float* decay, int T, int H, hipStream_t stream);
+// unit vectors of the q and k heads of qk [T, q (G d) | ... k at k_col (G d)] in place (q times q_scale); z [T, H d] turned
+// into decays exp(-exp(a_log[h]) softplus(z + dt_bias)) in place; beta[t, h] = sigmoid(rows[t, b_col + h])
+int alice_delta_prepare(float* qk, int qk_w, int k_col, int G, int d, float unit_eps, float q_scale, float* z,
+                        const float* dt_bias, const float* a_log, const float* rows, int row_w, int b_col, float* beta,
+                        int T, int H, hipStream_t stream);
+// The matrix-state recurrence over a step's tokens (delta 0: S = diag(a) S + k (b v)^T; 1: the delta rule), o to out
+// [T, H dv] float32; q and k are shared by groups of H / qk_heads heads; decay [T, H d] (decay_per_row) or [T, H].
+int alice_matrix_recurrence(const float* q, int q_w, int q_col, const float* k, int k_w, int k_col, const float* v, int v_w,
+                            int v_col, const float* decay, int decay_per_row, const float* b, const float* skip, float* out,
+                            const int* cu_seqlens, const int* slots, float* S, int n_seqs, int n_slots, int H, int qk_heads,
+                            int d, int dv, int delta, hipStream_t stream);
+// Rows of `width` in `parts` equal parts, each RMS-normed and multiplied by a weight (w_shared: of a part's length);
+// gate_act 1: times silu(gate) before the norm, 2: times sigmoid(gate) after it, 0: no gate.
+int alice_norm_gate(const float* x, int width, int parts, const float* gate, int gate_w, int gate_col, int gate_act,
+                    const float* w, int w_shared, float eps, void* out, int out_dtype, int T, hipStream_t stream);
+// Router of a mixture of experts: dense weights [T, E] from logits [T, E] (+ bias): softmax over the `top` largest,
+// zero elsewhere; and y[t, e F + j] = x[t, e F + j] w[t, e].  See experts.hip.
+int alice_route_topk(const float* z, const float* bias, float* w, int T, int E, int top, hipStream_t stream);
+int alice_scale_columns(const void* x, int x_dtype, const float* w, void* y, int y_dtype, int T, int E, int F, hipStream_t stream);
 // Latent attention (latent.hip): the cache row of a token is [latent (kv_rank) | rotated key part (rot_dim)], one kv head,
 // row-major pages; the first kv_rank dimensions of a row are also its value.
 int alice_latent_prepare(const float* rows, int row_width, int q_rank, int kv_rank, int rot_dim, const float* w_q,

@@ -8,14 +8,38 @@
 // v cos a + u sin a), a = p * f_i, from tables [positions, R/2].  With value tables [positions, dv/2] every value
 // head is turned the same way over all its dv dimensions by its own position (the attention kernel turns the
 // head's output back by the query's position).
+//
+// With norm weights the q columns (all heads together) and the k columns (likewise) are each divided by their root
+// mean square over the whole projection, eps inside the root, and multiplied by a weight of that length, after the
+// bias and before the rotation; projection_rms_kernel finds the two factors of every token first, in 32-bit.
 #include "common.h"
 #include "alice_hip.h"
 #include "kv_layout.h"
 
 namespace {
 
+// inv[t, part] = 1 / sqrt(mean over the part's columns of (row + bias)^2 + eps); part 0: the q columns [0, n_q),
+// part 1: the k columns [n_q, n_q + n_k).
+template <typename TI>
+__global__ __launch_bounds__(256) void projection_rms_kernel(const TI* __restrict__ rows, int row_w, const float* __restrict__ bias,
+                                                             float* __restrict__ inv, int n_q, int n_k, float eps) {
+  __shared__ float red[17];
+  const int t = blockIdx.x, part = blockIdx.y;
+  const int c0 = part ? n_q : 0, n = part ? n_k : n_q;
+  const TI* row = rows + (size_t)t * row_w;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < n; c += blockDim.x) {
+    float x = load_f32(row, (size_t)c0 + c);
+    if (bias) x += bias[c0 + c];
+    ss = fmaf(x, x, ss);
+  }
+  ss = block_sum(ss, red);
+  if (threadIdx.x == 0) inv[(size_t)t * 2 + part] = 1.f / sqrtf(ss / (float)n + eps);
+}
+
 template <typename TI, typename TO>
 __global__ void qkv_prepare_kernel(const TI* __restrict__ rows, int row_w, const float* __restrict__ bias,
+                                   const float* __restrict__ norm_w, const float* __restrict__ inv_rms,
                                    TO* __restrict__ q_out, TO* __restrict__ k_pool, TO* __restrict__ v_pool,
                                    const float* __restrict__ cos_t, const float* __restrict__ sin_t, int R, int interleaved,
                                    const float* __restrict__ vcos, const float* __restrict__ vsin,
@@ -38,10 +62,12 @@ __global__ void qkv_prepare_kernel(const TI* __restrict__ rows, int row_w, const
     TO* dst = is_q ? q_out + ((size_t)t * nH + h) * d
                    : k_pool + (((size_t)page * nKV + (h - nH)) * page_size + tp) * d;
     const int half = R >> 1;
+    const float inv = norm_w ? inv_rms[(size_t)t * 2 + (is_q ? 0 : 1)] : 1.f;
     for (int i = threadIdx.x; i < half; i += blockDim.x) {
       const int e0 = interleaved ? 2 * i : i, e1 = interleaved ? 2 * i + 1 : i + half;
       float x0 = load_f32(row, col0 + e0), x1 = load_f32(row, col0 + e1);
       if (bias) { x0 += bias[col0 + e0]; x1 += bias[col0 + e1]; }
+      if (norm_w) { x0 = x0 * inv * norm_w[col0 + e0]; x1 = x1 * inv * norm_w[col0 + e1]; }
       float y0, y1;
       rotate_pair(x0, x1, cos_t[(size_t)pos * half + i], sin_t[(size_t)pos * half + i], y0, y1);
       store_f32(dst, e0, y0);
@@ -50,6 +76,7 @@ __global__ void qkv_prepare_kernel(const TI* __restrict__ rows, int row_w, const
     for (int e = R + threadIdx.x; e < d; e += blockDim.x) {
       float x = load_f32(row, col0 + e);
       if (bias) x += bias[col0 + e];
+      if (norm_w) x = x * inv * norm_w[col0 + e];
       store_f32(dst, e, x);
     }
   } else if (page >= 0) {
@@ -93,8 +120,10 @@ extern "C" int alice_qkv_prepare(const void* rows, int rows_dtype, int row_width
                                  void* v_pool, int out_dtype, const float* cos_t, const float* sin_t, int rotary_dim,
                                  int interleaved, const float* vcos, const float* vsin, const int* positions,
                                  const int* seq_of_token, const int* block_table, int bt_stride, int T, int nH, int nKV,
-                                 int d, int dv, int page_size, int n_pages, hipStream_t stream) {
+                                 int d, int dv, int page_size, int n_pages, const float* norm_w, float norm_eps, float* inv_rms,
+                                 hipStream_t stream) {
   ALICE_CHECK(dtype_ok(rows_dtype) && dtype_ok(out_dtype), "qkv_prepare: unknown dtype");
+  ALICE_CHECK(norm_w == nullptr || (inv_rms != nullptr && norm_eps > 0.f), "qkv_prepare: the projection norm needs its workspace and a positive eps");
   ALICE_CHECK(rows_dtype == DT_F32 || rows_dtype == out_dtype, "qkv_prepare: rows are float32 or in the outputs' dtype");
   ALICE_CHECK(T >= 0 && nH >= 1 && nKV >= 0 && d >= 1 && dv >= 1, "qkv_prepare: bad sizes T=%d nH=%d nKV=%d d=%d dv=%d", T, nH, nKV, d, dv);
   ALICE_CHECK(rotary_dim >= 0 && rotary_dim <= d && rotary_dim % 2 == 0, "qkv_prepare: rotated width %d must be even and at most %d", rotary_dim, d);
@@ -108,8 +137,14 @@ extern "C" int alice_qkv_prepare(const void* rows, int rows_dtype, int row_width
   if (T == 0) return 0;
   dim3 grid(T, nH + (k_pool ? 2 * nKV : 0));
   const int threads = 64;
+  if (norm_w) {
+    dim3 g0(T, k_pool ? 2 : 1);
+    if (rows_dtype == DT_F32) projection_rms_kernel<float><<<g0, 256, 0, stream>>>((const float*)rows, row_width, bias, inv_rms, nH * d, k_pool ? nKV * d : 0, norm_eps);
+    else projection_rms_kernel<bf16_t><<<g0, 256, 0, stream>>>((const bf16_t*)rows, row_width, bias, inv_rms, nH * d, k_pool ? nKV * d : 0, norm_eps);
+    ALICE_LAUNCH_CHECK();
+  }
 #define GO(TI, TO)                                                                                                          \
-  qkv_prepare_kernel<TI, TO><<<grid, threads, 0, stream>>>((const TI*)rows, row_width, bias, (TO*)q_out, (TO*)k_pool, (TO*)v_pool, \
+  qkv_prepare_kernel<TI, TO><<<grid, threads, 0, stream>>>((const TI*)rows, row_width, bias, norm_w, inv_rms, (TO*)q_out, (TO*)k_pool, (TO*)v_pool, \
       cos_t, sin_t, rotary_dim, interleaved, vcos, vsin, positions, seq_of_token, block_table, bt_stride, nH, nKV, d, dv, page_size, n_pages)
   if (rows_dtype == DT_F32 && out_dtype == DT_F32) GO(float, float);
   else if (rows_dtype == DT_F32) GO(float, bf16_t);

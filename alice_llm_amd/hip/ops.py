@@ -18,7 +18,7 @@ from ..csrc import build as _build
 EPI_NONE, EPI_GEGLU, EPI_SOFTCAP = 0, 1, 2
 LAYOUT_ROW, LAYOUT_FRAG16 = 0, 1
 LINEAR_AUTO, LINEAR_GENERIC, LINEAR_SKINNY, LINEAR_MFMA, LINEAR_TILED_W16, LINEAR_TILED_W32 = 0, 1, 2, 3, 4, 5
-ABI_VERSION = 11
+ABI_VERSION = 12
 GATED_SILU = -1.0        # epi_param of EPI_GEGLU that picks silu(gate) * up
 UNARY_RELU2 = -1.0       # epi_param of EPI_SOFTCAP that picks the square of max(y, 0) instead of the capped form
 
@@ -65,7 +65,14 @@ def _declare(lib) -> None:
         "alice_attention_split_supported": [I, I, I, I, I],
         "alice_attention_split_runs": [I],
         "alice_mix_heads": [P, P, P, I, F, P, I, I, I, I, I, I, P],
-        "alice_qkv_prepare": [P, I, I, P, P, P, P, I, P, P, I, I, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
+        "alice_qkv_prepare": [P, I, I, P, P, P, P, I, P, P, I, I, P, P, P, P, P, I, I, I, I, I, I, I, I, P, F, P, P],
+        "alice_short_conv": [P, I, I, I, I, P, P, P, P, I, P, P, P, I, I, P],
+        "alice_ssm_prepare": [P, I, I, P, P, P, P, I, I, P],
+        "alice_delta_prepare": [P, I, I, I, I, F, F, P, P, P, P, I, I, P, I, I, P],
+        "alice_matrix_recurrence": [P, I, I, P, I, I, P, I, I, P, I, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
+        "alice_norm_gate": [P, I, I, P, I, I, I, P, I, F, P, I, I, P],
+        "alice_route_topk": [P, P, P, I, I, I, P],
+        "alice_scale_columns": [P, I, P, P, I, I, I, I, P],
         "alice_add_rows": [P, P, P, I, I, P],
         "alice_latent_prepare": [P, I, I, I, I, P, P, F, P, P, P, P, P, I, I, I, P, P, I, I, P],
         "alice_heads_linear": [P, I, L, I, P, I, P, I, L, I, I, I, I, I, I, P, P, P, P],
@@ -705,11 +712,15 @@ def qkv_prepare(rows: torch.Tensor, bias: Optional[torch.Tensor], q_out: torch.T
                 block_table: Optional[torch.Tensor], *, num_heads: int, num_kv_heads: int, head_dim: int,
                 value_head_dim: int, max_position: int, cos: Optional[torch.Tensor] = None,
                 sin: Optional[torch.Tensor] = None, rotary_dim: int = 0, interleaved: bool = True,
-                value_cos: Optional[torch.Tensor] = None, value_sin: Optional[torch.Tensor] = None) -> None:
+                value_cos: Optional[torch.Tensor] = None, value_sin: Optional[torch.Tensor] = None,
+                norm_weight: Optional[torch.Tensor] = None, norm_eps: float = 0.0) -> None:
     """From the rows [q | k | v | ...] of a fused projection (float32, or q_out's dtype): bias [>= q, k, v columns]
     added, q and k heads rotated over their first rotary_dim dimensions in pairs ((2i, 2i + 1) if interleaved, else
     (i, i + rotary_dim / 2)) from tables [positions, rotary_dim / 2], values turned over all their dimensions where
-    value tables [positions, dv / 2] are given; q to q_out, k and v into the row-major pools at their positions."""
+    value tables [positions, dv / 2] are given; q to q_out, k and v into the row-major pools at their positions.
+    norm_weight: float32 [q columns + k columns (where a cache is written)]: after the bias and before the rotation, the q
+    columns (all heads together) and the k columns are each divided by their root mean square over the whole projection
+    (norm_eps inside the root) and multiplied by this weight."""
     T = rows.shape[0]
     dt = q_out.dtype
     d, dv = head_dim, value_head_dim
@@ -745,11 +756,19 @@ def qkv_prepare(rows: torch.Tensor, bias: Optional[torch.Tensor], q_out: torch.T
         if block_table.dim() != 2 or max_position // page_size >= block_table.shape[1]:
             raise HipLibraryError(f"position {max_position} is beyond the block table")
         bt_stride = block_table.shape[1]
+    inv_rms = None
+    if norm_weight is not None:
+        n_norm = num_heads * d + (num_kv_heads * d if k_pool is not None else 0)
+        _dev(norm_weight, "norm_weight", torch.float32, (n_norm,))
+        if not norm_eps > 0:
+            raise HipLibraryError("the projection norm needs a positive eps")
+        inv_rms = torch.empty((T, 2), dtype=torch.float32, device=rows.device)
     _call("alice_qkv_prepare", rows.data_ptr(), dtype_code(rows.dtype), rows.shape[1], _opt(bias, "bias"), q_out.data_ptr(),
           _opt(k_pool, "k_pool"), _opt(v_pool, "v_pool"), dtype_code(dt), _opt(cos, "cos"), _opt(sin, "sin"),
           int(rotary_dim if cos is not None else 0), int(interleaved), _opt(value_cos, "value_cos"), _opt(value_sin, "value_sin"),
           positions.data_ptr(), _opt(seq_of_token, "seq_of_token"), _opt(block_table, "block_table"), bt_stride, T,
-          num_heads, num_kv_heads if k_pool is not None else 0, d, dv, page_size, n_pages, _stream())
+          num_heads, num_kv_heads if k_pool is not None else 0, d, dv, page_size, n_pages,
+          _opt(norm_weight, "norm_weight"), float(norm_eps), _opt(inv_rms, "inv_rms"), _stream())
 
 
 def add_rows(x: torch.Tensor, rows: Optional[torch.Tensor], vector: Optional[torch.Tensor]) -> None:
@@ -946,6 +965,153 @@ def gla(rows: torch.Tensor, z: torch.Tensor, z_bias: torch.Tensor, norm_w: torch
           float(q_scale), float(out_scale), norm_w.data_ptr(), dtype_code(norm_w.dtype), float(eps), out.data_ptr(), dtype_code(out.dtype),
           _opt(work, "work"), ctx.cu_seqlens.data_ptr(), ctx.slots.data_ptr(), S.data_ptr(), T, int(ctx.n_seqs), int(n_slots),
           H, d, dv, int(columns_per_block), _stream())
+
+
+# ------------------------------------------------------------------------------------ recurrent mixers
+
+SHORT_CONV_MAX_TAPS = 16        # the most taps the short convolution takes
+RECURRENCE_MAX_KEY_DIM = 256    # the largest key size the matrix recurrence keeps in registers
+ROUTER_MAX_EXPERTS = 1024       # the most experts the router's kernel ranks
+
+
+def _step_arrays(ctx) -> None:
+    _dev(ctx.cu_seqlens, "cu_seqlens", torch.int32)
+    _dev(ctx.slots, "slots", torch.int32)
+    if ctx.cu_seqlens.numel() < ctx.n_seqs + 1 or ctx.slots.numel() < ctx.n_seqs:
+        raise HipLibraryError("cu_seqlens and slots are too short for the step's sequences")
+
+
+def short_conv(rows: torch.Tensor, col0: int, weight: torch.Tensor, bias: Optional[torch.Tensor], state: Optional[torch.Tensor],
+               out: torch.Tensor, ctx, *, silu: bool = True) -> None:
+    """out[t, c] = act(bias[c] + sum_j weight[c, j] x[t - (taps - 1) + j, c]) with x = rows[:, col0 + c] (float32), over the
+    tokens of the token's own sequence; what lies before the step comes from state float32 [slots, channels, taps - 1]
+    (the last inputs of the sequence's earlier steps, zeros at its start), which then takes the step's last inputs."""
+    T = rows.shape[0]
+    if weight.dim() != 2:
+        raise HipLibraryError("weight must be [channels, taps]")
+    C, taps = weight.shape
+    _dev(rows, "rows", torch.float32)
+    if rows.dim() != 2 or col0 < 0 or col0 + C > rows.shape[1]:
+        raise HipLibraryError(f"rows of {tuple(rows.shape)} are too short for {C} channels from column {col0}")
+    _dev(weight, "weight", torch.float32)
+    _opt(bias, "bias", torch.float32, (C,))
+    _dev(out, "out", torch.float32, (T, C))
+    _step_arrays(ctx)
+    _dev(ctx.seq_of_token, "seq_of_token", torch.int32)
+    if ctx.seq_of_token.numel() < T:
+        raise HipLibraryError("seq_of_token is too short for the step")
+    if taps > 1:
+        if state is None or state.dim() != 3 or tuple(state.shape[1:]) != (C, taps - 1):
+            raise HipLibraryError(f"state must be [slots, {C}, {taps - 1}]")
+        _dev(state, "state", torch.float32)
+    _call("alice_short_conv", rows.data_ptr(), rows.shape[1], int(col0), C, taps, weight.data_ptr(), _opt(bias, "bias"),
+          None if taps == 1 else state.data_ptr(), out.data_ptr(), int(bool(silu)), ctx.cu_seqlens.data_ptr(),
+          ctx.seq_of_token.data_ptr(), ctx.slots.data_ptr(), T, int(ctx.n_seqs), _stream())
+
+
+def ssm_prepare(rows: torch.Tensor, dt_col: int, dt_bias: torch.Tensor, a_log: torch.Tensor, step: torch.Tensor,
+                decay: torch.Tensor) -> None:
+    """step = softplus(rows[:, dt_col + h] + dt_bias[h]); decay = exp(-exp(a_log[h]) * step); float32 [T, heads] each."""
+    T, H = step.shape
+    _dev(rows, "rows", torch.float32)
+    _dev(dt_bias, "dt_bias", torch.float32, (H,))
+    _dev(a_log, "a_log", torch.float32, (H,))
+    _dev(step, "step", torch.float32)
+    _dev(decay, "decay", torch.float32, (T, H))
+    if rows.shape[0] != T or dt_col + H > rows.shape[1]:
+        raise HipLibraryError("rows do not hold the step sizes")
+    _call("alice_ssm_prepare", rows.data_ptr(), rows.shape[1], int(dt_col), dt_bias.data_ptr(), a_log.data_ptr(), step.data_ptr(),
+          decay.data_ptr(), T, H, _stream())
+
+
+def delta_prepare(qk: torch.Tensor, k_col: int, z: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, rows: torch.Tensor,
+                  b_col: int, beta: torch.Tensor, *, qk_heads: int, heads: int, head_dim: int, unit_eps: float, q_scale: float) -> None:
+    """In place: the q heads (columns 0 .. qk_heads * d of qk) and the k heads (from k_col) become unit vectors
+    x / sqrt(sum x^2 + unit_eps), q also times q_scale; z [T, heads * d] becomes exp(-exp(a_log[h]) softplus(z + dt_bias));
+    beta[t, h] = sigmoid(rows[t, b_col + h])."""
+    T = qk.shape[0]
+    G, H, d = qk_heads, heads, head_dim
+    _dev(qk, "qk", torch.float32)
+    _dev(z, "z", torch.float32, (T, H * d))
+    _dev(dt_bias, "dt_bias", torch.float32, (H * d,))
+    _dev(a_log, "a_log", torch.float32, (H,))
+    _dev(rows, "rows", torch.float32)
+    _dev(beta, "beta", torch.float32, (T, H))
+    if rows.shape[0] != T or b_col + H > rows.shape[1] or k_col < G * d or k_col + G * d > qk.shape[1]:
+        raise HipLibraryError("the rows are too short for the heads")
+    _call("alice_delta_prepare", qk.data_ptr(), qk.shape[1], int(k_col), G, d, float(unit_eps), float(q_scale), z.data_ptr(),
+          dt_bias.data_ptr(), a_log.data_ptr(), rows.data_ptr(), rows.shape[1], int(b_col), beta.data_ptr(), T, H, _stream())
+
+
+def matrix_recurrence(q, q_col: int, k, k_col: int, v, v_col: int, decay: torch.Tensor, b: torch.Tensor, skip: Optional[torch.Tensor],
+                      out: torch.Tensor, ctx, S: torch.Tensor, *, heads: int, qk_heads: int, head_dim: int, value_head_dim: int,
+                      delta: bool, decay_per_channel: bool) -> None:
+    """The recurrence of a matrix state a head over a step (`ctx` gives cu_seqlens, slots, n_seqs), all float32:
+    delta False: S = diag(a) S + k (b v)^T; True: S = diag(a) S, u = b (v - S^T k), S += k u^T; then o = S^T q (+ skip[h] v).
+    q, k: rows with the heads' columns from q_col / k_col, shared by groups of heads / qk_heads heads; v: rows with
+    heads * dv columns from v_col; decay: [T, heads * d] (decay_per_channel) or [T, heads]; b: [T, heads]; S: [slots, heads, d, dv]; out: [T, heads * dv]."""
+    H, d, dv = heads, head_dim, value_head_dim
+    T = out.shape[0]
+    for t_, nm in ((q, "q"), (k, "k"), (v, "v")):
+        _dev(t_, nm, torch.float32)
+        if t_.dim() != 2 or t_.shape[0] != T:
+            raise HipLibraryError(f"{nm} must be [T, width]")
+    if q_col + qk_heads * d > q.shape[1] or k_col + qk_heads * d > k.shape[1] or v_col + H * dv > v.shape[1]:
+        raise HipLibraryError("the rows are too short for the heads")
+    per_row = bool(decay_per_channel)
+    _dev(decay, "decay", torch.float32, (T, H * d) if per_row else (T, H))
+    _dev(b, "b", torch.float32, (T, H))
+    _opt(skip, "skip", torch.float32, (H,))
+    _dev(out, "out", torch.float32, (T, H * dv))
+    _step_arrays(ctx)
+    n_slots = S.shape[0]
+    _dev(S, "S", torch.float32, (n_slots, H, d, dv))
+    _call("alice_matrix_recurrence", q.data_ptr(), q.shape[1], int(q_col), k.data_ptr(), k.shape[1], int(k_col), v.data_ptr(),
+          v.shape[1], int(v_col), decay.data_ptr(), int(per_row), b.data_ptr(), _opt(skip, "skip"), out.data_ptr(),
+          ctx.cu_seqlens.data_ptr(), ctx.slots.data_ptr(), S.data_ptr(), int(ctx.n_seqs), int(n_slots), H, int(qk_heads), d, dv,
+          int(bool(delta)), _stream())
+
+
+def norm_gate(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, *, parts: int, eps: float, weight_shared: bool,
+              gate: Optional[torch.Tensor] = None, gate_col: int = 0, gate_act: Optional[str] = None) -> None:
+    """Rows of x (float32 [T, width]) in `parts` equal parts, each divided by its root mean square (eps inside the root)
+    and multiplied by weight (float32, of the row's length, or with weight_shared of a part's length, the same for every part).
+    gate_act "silu": times silu(gate[:, gate_col + .]) before the norm; "sigmoid": times sigmoid(.) after it."""
+    T, width = x.shape
+    _dev(x, "x", torch.float32)
+    _dev(out, "out", None, (T, width))
+    if width % parts:
+        raise HipLibraryError(f"{parts} parts must divide the width {width}")
+    _dev(weight, "weight", torch.float32, (width // parts if weight_shared else width,))
+    act = {None: 0, "silu": 1, "sigmoid": 2}[gate_act]
+    if act:
+        _dev(gate, "gate", torch.float32)
+        if gate.dim() != 2 or gate.shape[0] != T or gate_col + width > gate.shape[1]:
+            raise HipLibraryError("the gate rows are too short")
+    _call("alice_norm_gate", x.data_ptr(), width, int(parts), _opt(gate, "gate") if act else None, gate.shape[1] if act else 0,
+          int(gate_col), act, weight.data_ptr(), int(bool(weight_shared)), float(eps), out.data_ptr(),
+          dtype_code(out.dtype), T, _stream())
+
+
+def route_topk(logits: torch.Tensor, bias: Optional[torch.Tensor], weights: torch.Tensor, top: int) -> None:
+    """weights[t] = softmax over the `top` largest of logits[t] + bias at their places, zero elsewhere; float32 [T, experts]."""
+    T, E = logits.shape
+    _dev(logits, "logits", torch.float32)
+    _opt(bias, "bias", torch.float32, (E,))
+    _dev(weights, "weights", torch.float32, (T, E))
+    _call("alice_route_topk", logits.data_ptr(), _opt(bias, "bias"), weights.data_ptr(), T, E, int(top), _stream())
+
+
+def scale_columns(x: torch.Tensor, weights: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t, e * F + j] = x[t, e * F + j] * weights[t, e] for x [T, experts * F] and float32 weights [T, experts]."""
+    T, E = weights.shape
+    _dev(x, "x", None, (T, x.shape[1]))
+    if x.shape[1] % E:
+        raise HipLibraryError("the row must hold a whole number of columns an expert")
+    _dev(weights, "weights", torch.float32)
+    _dev(out, "out", None, tuple(x.shape))
+    _call("alice_scale_columns", x.data_ptr(), dtype_code(x.dtype), weights.data_ptr(), out.data_ptr(), dtype_code(out.dtype),
+          T, E, x.shape[1] // E, _stream())
 
 
 def fragment_layout_supported(rows: int, k_in: int, epilogue: int) -> bool:

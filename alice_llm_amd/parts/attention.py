@@ -21,7 +21,14 @@ until the bias is added and the rotation done):
                   sequence's position 0 (the cache gives the pages of finished chunks back like a window's)
   keep_first      beside its window a query sees the first that many positions (the cache keeps their pages)
   sink            one learned number a head ("sink") whose exponential joins the softmax's denominator; it has no
-                  key and no value
+                  key and no value.  "zero": the number is 0 for every head and no tensor is read (the denominator is
+                  one more than the sum of the exponentials)
+  qk_norm         "projection": q (all heads together) and k (likewise) are each divided by their root mean square over
+                  the whole projection (qk_norm_eps inside the root) and multiplied by a weight of that length ("q_norm",
+                  "k_norm"), after the bias and before the rotation
+  output_bias     the output matrix has a bias ("o_bias")
+  own_keys        False: the mixer has no k and v matrices (nor their biases and norm); it reads the keys and values that
+                  another run of the schedule cached and brings its own queries, gate and output matrix
   talk            the heads' softmax weights are mixed by a learned matrix ("talk" [heads, heads]) before they meet
                   the values: weight_h <- sum_g talk[h, g] weight_g, head h keeping its own kv head's values
   output_gate     "elementwise": sigmoid of a projection of the mixer's input ("g" [heads * value size, width]) times
@@ -50,8 +57,9 @@ class Attention(Part):
                  window: Optional[int] = None, position: Optional[str] = None,
                  score_bias_slopes: Optional[Sequence[float]] = None, value_head_dim: Optional[int] = None,
                  output_gate: Optional[str] = None, tensor_names: Optional[Dict[str, str]] = None,
-                 bias: bool = False, chunk: Optional[int] = None, keep_first: int = 0, sink: bool = False,
-                 talk: bool = False, output_scale: float = 1.0):
+                 bias: bool = False, chunk: Optional[int] = None, keep_first: int = 0, sink=False,
+                 talk: bool = False, output_scale: float = 1.0, qk_norm: Optional[str] = None, qk_norm_eps: float = 1e-6,
+                 output_bias: bool = False, own_keys: bool = True):
         if num_heads % num_kv_heads:
             raise ValueError(f"num_kv_heads {num_kv_heads} must divide num_heads {num_heads}")
         if not 1 <= head_dim <= ops.ATTENTION_MAX_HEAD_DIM:
@@ -82,22 +90,36 @@ class Attention(Part):
         self.output_gate = output_gate
         self.n_gate = {None: 0, "head": num_heads, "elementwise": num_heads * self.dv}[output_gate]
         self.bias, self.chunk, self.keep_first = bool(bias), chunk, int(keep_first)
+        if sink not in (False, True, None, "zero"):
+            raise ValueError(f"attention: sink '{sink}' is not known (False, True or 'zero')")
+        if qk_norm not in (None, "projection"):
+            raise ValueError(f"attention: qk_norm '{qk_norm}' is not known (None or 'projection')")
         self.has_sink, self.has_talk, self.output_scale = bool(sink), bool(talk), float(output_scale)
+        self.zero_sink = sink == "zero"
+        self.qk_norm, self.qk_norm_eps = qk_norm, float(qk_norm_eps)
+        self.output_bias, self.own_keys = bool(output_bias), bool(own_keys)
         pairs = getattr(self.position, "value_cos", "absent") != "absent"          # a rope_pairs encoding
         # the mixers made by the further arguments: float32 projection sums, bias and rotation in one kernel, the
         # 32-bit attention kernel with its further masks over a row-major cache
         self.extended = bool(bias or chunk or keep_first or sink or talk or output_gate == "elementwise"
-                             or output_scale != 1.0 or pairs)
+                             or output_scale != 1.0 or pairs or qk_norm or output_bias or not own_keys)
         if self.extended and softcap is not None and talk:
             raise ValueError("attention: mixed heads take no softcap")
         self.names = dict({"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
-                           "g": "g_proj.weight", "sink": "sink", "talk": "talk"}, **(tensor_names or {}))
+                           "g": "g_proj.weight", "sink": "sink", "talk": "talk", "q_norm": "q_norm.weight",
+                           "k_norm": "k_norm.weight", "o_bias": "o_proj.bias"}, **(tensor_names or {}))
         self._bias_parts: Dict[str, torch.Tensor] = {}
         self.qkv_bias: Optional[torch.Tensor] = None
         self.sink: Optional[torch.Tensor] = None
         self.talk: Optional[torch.Tensor] = None
-        self.q_dim, self.kv_dim, self.v_dim = num_heads * head_dim, num_kv_heads * head_dim, num_kv_heads * self.dv
+        self.q_dim = num_heads * head_dim
+        # (a mixer without keys of its own has no k and v columns in its projection)
+        self.kv_dim, self.v_dim = (num_kv_heads * head_dim, num_kv_heads * self.dv) if self.own_keys else (0, 0)
         self.o_in = num_heads * self.dv
+        self.o_bias: Optional[torch.Tensor] = None
+        self._norm_parts: Dict[str, torch.Tensor] = {}
+        self.qk_norm_w: Optional[torch.Tensor] = None
+        self._mats = "q" + ("kv" if self.own_keys else "") + ("g" if self.n_gate else "")
         # one fused projection: all q heads, the k heads, the v heads, then the gate numbers
         self.qkv = Linear(hidden_size, self.q_dim + self.kv_dim + self.v_dim + self.n_gate, precision)
         self.o = Linear(self.o_in, hidden_size, precision)
@@ -111,17 +133,25 @@ class Attention(Part):
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         n = self.names
-        specs = {n["q"]: ParamSpec((self.q_dim, self.H)),
-                 n["k"]: ParamSpec((self.kv_dim, self.H)),
-                 n["v"]: ParamSpec((self.v_dim, self.H)),
-                 n["o"]: ParamSpec((self.H, self.o_in))}
+        specs = {n["q"]: ParamSpec((self.q_dim, self.H))}
+        if self.own_keys:
+            specs[n["k"]] = ParamSpec((self.kv_dim, self.H))
+            specs[n["v"]] = ParamSpec((self.v_dim, self.H))
+        specs[n["o"]] = ParamSpec((self.H, self.o_in))
         if self.n_gate:
             specs[n["g"]] = ParamSpec((self.n_gate, self.H))
         if self.bias:
             specs[n["q"] + ".b"] = ParamSpec((self.q_dim,), init_std=0.1)
-            specs[n["k"] + ".b"] = ParamSpec((self.kv_dim,), init_std=0.1)
-            specs[n["v"] + ".b"] = ParamSpec((self.v_dim,), init_std=0.1)
-        if self.has_sink:
+            if self.own_keys:
+                specs[n["k"] + ".b"] = ParamSpec((self.kv_dim,), init_std=0.1)
+                specs[n["v"] + ".b"] = ParamSpec((self.v_dim,), init_std=0.1)
+        if self.qk_norm:
+            specs[n["q_norm"]] = ParamSpec((self.q_dim,), init_std=0.3)
+            if self.own_keys:
+                specs[n["k_norm"]] = ParamSpec((self.kv_dim,), init_std=0.3)
+        if self.output_bias:
+            specs[n["o_bias"]] = ParamSpec((self.H,), init_std=0.1)
+        if self.has_sink and not self.zero_sink:
             specs[n["sink"]] = ParamSpec((self.nH,), init_std=1.0)
         if self.has_talk:
             specs[n["talk"]] = ParamSpec((self.nH, self.nH), init_std=0.3)
@@ -137,11 +167,15 @@ class Attention(Part):
     def assign(self, name: str, tensor: torch.Tensor) -> None:
         if name == self.names["o"]:
             self.o.load(tensor)
-        elif name in [self.names[c] for c in ("qkvg" if self.n_gate else "qkv")]:
+        elif name in [self.names[c] for c in self._mats]:
             self._parts[name] = tensor
-        elif self.bias and name in [self.names[c] + ".b" for c in "qkv"]:
+        elif self.bias and name in [self.names[c] + ".b" for c in self._mats if c != "g"]:
             self._bias_parts[name] = tensor
-        elif self.has_sink and name == self.names["sink"]:
+        elif self.qk_norm and name in (self.names["q_norm"], self.names["k_norm"]):
+            self._norm_parts[name] = tensor
+        elif self.output_bias and name == self.names["o_bias"]:
+            self.o_bias = tensor.float().contiguous()
+        elif self.has_sink and not self.zero_sink and name == self.names["sink"]:
             self.sink = tensor.float().contiguous()
         elif self.has_talk and name == self.names["talk"]:
             self.talk = tensor.float().contiguous()
@@ -149,7 +183,7 @@ class Attention(Part):
             raise KeyError(name)
 
     def finalize(self) -> None:
-        mats = [self.precision.matrix(self._parts.pop(self.names[c])) for c in ("qkvg" if self.n_gate else "qkv")]
+        mats = [self.precision.matrix(self._parts.pop(self.names[c])) for c in self._mats]
         if len({m.dtype for m in mats}) > 1:
             mats = [m.float() for m in mats]                # kept as stored, one of them in 32-bit: the fused matrix is 32-bit
         w = torch.cat(mats, dim=0)                          # rows: all q heads, then k heads, then v heads, then the gates
@@ -158,7 +192,12 @@ class Attention(Part):
         order = getattr(self.position, "projection_row_order", lambda *a: None)(self.nH, self.nKV, self.d)
         self.pair_order = order is not None and self.dv == self.d and not self.n_gate and not self.extended
         if self.bias:
-            self.qkv_bias = torch.cat([self._bias_parts.pop(self.names[c] + ".b").float() for c in "qkv"]).contiguous()
+            self.qkv_bias = torch.cat([self._bias_parts.pop(self.names[c] + ".b").float() for c in self._mats if c != "g"]).contiguous()
+        if self.qk_norm:
+            self.qk_norm_w = torch.cat([self._norm_parts.pop(self.names[c]).float()
+                                        for c in (("q_norm", "k_norm") if self.own_keys else ("q_norm",))]).contiguous()
+        if self.zero_sink:
+            self.sink = torch.zeros(self.nH, dtype=torch.float32, device=w.device)
         if self.pair_order:
             w = w[order.to(w.device)]
         self.qkv.load(w)
@@ -224,12 +263,18 @@ class Attention(Part):
         q = torch.empty((T, self.q_dim), dtype=act, device=dev)
         pos = self.position
         write = cache is not None and cache.writable
+        if write and not self.own_keys:
+            raise RuntimeError("attention: a mixer without keys of its own reads the cache of another run of the schedule")
+        norm_w = self.qk_norm_w
+        if norm_w is not None and self.own_keys and not write:
+            norm_w = norm_w[:self.q_dim]                      # the keys are another run's: only the queries are normed here
         ops.qkv_prepare(rows, self.qkv_bias, q, cache.k if write else None, cache.v if write else None, ctx.positions,
                         ctx.seq_of_token if write else None, cache.block_table if write else None,
                         num_heads=self.nH, num_kv_heads=self.nKV, head_dim=self.d, value_head_dim=self.dv,
                         max_position=ctx.max_position, cos=getattr(pos, "cos", None), sin=getattr(pos, "sin", None),
                         rotary_dim=getattr(pos, "rotary_dim", 0), interleaved=getattr(pos, "interleaved", True),
-                        value_cos=getattr(pos, "value_cos", None), value_sin=getattr(pos, "value_sin", None))
+                        value_cos=getattr(pos, "value_cos", None), value_sin=getattr(pos, "value_sin", None),
+                        norm_weight=norm_w, norm_eps=self.qk_norm_eps)
         gate = None
         if self.n_gate:
             g0 = self.q_dim + self.kv_dim + self.v_dim
@@ -272,4 +317,8 @@ class Attention(Part):
             ops.mix_heads(per, self.talk, gate, out, full_precision=self.precision.full, out_scale=self.output_scale)
         else:
             attend(out, None, gate=gate, gate_per_element=self.output_gate == "elementwise", out_scale=self.output_scale)
-        return self.o(out, torch.float32, allow_partials=True)
+        if self.o_bias is None:
+            return self.o(out, torch.float32, allow_partials=True)
+        y = self.o(out, torch.float32)
+        ops.add_rows(y, None, self.o_bias)
+        return y

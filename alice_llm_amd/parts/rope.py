@@ -8,6 +8,7 @@ same pass, which saves one trip through memory for k.
 """
 from __future__ import annotations
 
+import math
 from typing import Optional
 
 import torch
@@ -86,11 +87,17 @@ class RotaryPairs(Part):
     turned too, over all their dimensions and with frequencies of their own, theta^(-2m / value_dim), by their
     own position, and the attention kernel turns every head's output back by the query's position (so that a
     value enters the output turned by the distance).  The tables are made on the host in 64-bit and kept in
-    32-bit; the attention mixer hands them to its kernels (`cos`, `sin`, `value_cos`, `value_sin`)."""
+    32-bit; the attention mixer hands them to its kernels (`cos`, `sin`, `value_cos`, `value_sin`).
+
+    `scaling` (factor s, original length L, fast, slow) stretches the frequencies of the q and k rotation for
+    contexts beyond L, the slow ones most: with D(t) = R ln(L / (2 pi t)) / (2 ln theta), lo = max(floor D(fast), 0),
+    hi = min(ceil D(slow), R - 1) and r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), the frequency becomes
+    f_i / s * r_i + f_i (1 - r_i), and cos and sin are multiplied by 0.1 ln(s) + 1 (which the tables hold)."""
     graph_safe = True
 
     def __init__(self, precision: Precision, device, *, dim: int, theta: float, max_positions: int,
-                 rotary_dim: Optional[int] = None, value_dim: Optional[int] = None, interleaved: bool = True):
+                 rotary_dim: Optional[int] = None, value_dim: Optional[int] = None, interleaved: bool = True,
+                 scaling: Optional[dict] = None):
         self.dim = dim
         self.rotary_dim = dim if rotary_dim is None else int(rotary_dim)
         if self.rotary_dim % 2 or not 0 <= self.rotary_dim <= dim:
@@ -99,14 +106,30 @@ class RotaryPairs(Part):
             raise ValueError(f"turned values need an even size, found {value_dim}")
         self.theta, self.max_positions = float(theta), max_positions
         self.value_dim, self.interleaved = value_dim, bool(interleaved)
-        self.cos, self.sin = self._tables(self.rotary_dim, device) if self.rotary_dim else (None, None)
+        self.scaling = None if not scaling else {k: float(scaling[k]) for k in ("factor", "original", "fast", "slow")}
+        if self.scaling is not None and min(self.scaling.values()) <= 0:
+            raise ValueError(f"stretched frequencies need positive factor, original, fast and slow, found {self.scaling}")
+        self.cos, self.sin = self._tables(self.rotary_dim, device, self.scaling) if self.rotary_dim else (None, None)
         self.value_cos, self.value_sin = self._tables(value_dim, device) if value_dim else (None, None)
 
-    def _tables(self, width: int, device):
+    def frequencies(self, width: int, scaling: Optional[dict] = None):
+        """(the width / 2 frequencies in 64-bit, the factor of cos and sin)."""
         i = torch.arange(width // 2, dtype=torch.float64)
-        ang = torch.arange(self.max_positions, dtype=torch.float64)[:, None] * (self.theta ** (-2.0 * i / width))[None, :]
-        return (torch.cos(ang).to(torch.float32).to(device).contiguous(),
-                torch.sin(ang).to(torch.float32).to(device).contiguous())
+        f = self.theta ** (-2.0 * i / width)
+        if scaling is None:
+            return f, 1.0
+        s, L = scaling["factor"], scaling["original"]
+        at = lambda t: width * math.log(L / (2.0 * math.pi * t)) / (2.0 * math.log(self.theta))
+        lo = max(math.floor(at(scaling["fast"])), 0)
+        hi = min(math.ceil(at(scaling["slow"])), width - 1)
+        ramp = torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        return f / s * ramp + f * (1.0 - ramp), 0.1 * math.log(s) + 1.0
+
+    def _tables(self, width: int, device, scaling: Optional[dict] = None):
+        f, magnitude = self.frequencies(width, scaling)
+        ang = torch.arange(self.max_positions, dtype=torch.float64)[:, None] * f[None, :]
+        return ((torch.cos(ang) * magnitude).to(torch.float32).to(device).contiguous(),
+                (torch.sin(ang) * magnitude).to(torch.float32).to(device).contiguous())
 
 
 @POSITIONS.register("none")
