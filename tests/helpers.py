@@ -496,3 +496,146 @@ def pefitar_folder(name: str, seed: int = 0) -> str:
         save_file({k: v.contiguous() for k, v in tensors.items()}, os.path.join(folder, "model.safetensors"))
         _FOLDERS[key] = folder
     return _FOLDERS[key]
+
+
+# --------------------------------------------------------------------------- Vifirax test configurations
+# A: a state-space layer first (grouped B and C, four norm parts); attention with grouped kv heads, values twice the key
+#    size, a part of the head turned with stretched frequencies, a routed feed-forward (2 of 6); a delta-rule layer with
+#    grouped q and k and no feed-forward; an attention layer that reads the second layer's keys.
+# B: sizes that fit no tile (width 72, heads of 20 / 28 / 12); attention first with the whole head turned and no
+#    stretching, kv heads = heads; a routed feed-forward that uses every expert and one that uses a single one; a
+#    convolution of one tap (no convolution state); eps other than A's; no logit factor in the file.
+# C: sizes that suit the matrix cores; a delta-rule layer first with one q/k head for two heads and values wider than
+#    64; a state of 128 numbers a column; two attention layers that read another's keys, one without a feed-forward;
+#    an attention layer with no rotation at all.
+# D: two layers that read the first layer's keys; key sizes of the recurrences beyond 128; five taps; three query heads a
+#    kv head; three norm parts; a single delta-rule head.
+def _vx_rot(base, dims, scaling=None):
+    rot = {"base": base, "dims": dims}
+    if scaling is not None:
+        rot["scaling"] = dict(zip(("factor", "original", "fast", "slow"), scaling))
+    return rot
+
+
+def _vx_moe(experts, top, ff):
+    return {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+
+
+def _vx_a():
+    at = {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 32, "scale": 0.6, "rot": _vx_rot(100.0, 8, (4.0, 16, 8.0, 1.0))}
+    ss = {"heads": 4, "vdim": 16, "state": 8, "groups": 2, "norm_groups": 4, "conv": 4}
+    de = {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 8, "conv": 2, "decay_rank": 6, "gate_rank": 5}
+    return {"architecture": "Vifirax", "vocab": 97, "width": 64, "norm": {"eps": 1e-6}, "logit_scale": 0.37,
+            "layers": [{"type": "mamba2", "mixer": ss, "mlp": {"kind": "dense", "ff": 96}},
+                       {"type": "attention", "mixer": at, "mlp": _vx_moe(6, 2, 24)},
+                       {"type": "channel_delta", "mixer": de, "mlp": None},
+                       {"type": "attention", "mixer": dict(at, kv_from=1), "mlp": {"kind": "dense", "ff": 40}}]}
+
+
+def _vx_b():
+    at = {"heads": 3, "kv_heads": 3, "dim": 20, "vdim": 28, "scale": 0.5, "rot": _vx_rot(10000.0, 20)}
+    de = {"heads": 3, "kv_heads": 3, "dim": 12, "vdim": 20, "conv": 3, "decay_rank": 7, "gate_rank": 3}
+    ss = {"heads": 3, "vdim": 20, "state": 12, "groups": 3, "norm_groups": 1, "conv": 1}
+    return {"architecture": "Vifirax", "vocab": 130, "width": 72, "norm": {"eps": 1e-5},
+            "layers": [{"type": "attention", "mixer": at, "mlp": _vx_moe(5, 5, 18)},
+                       {"type": "channel_delta", "mixer": de, "mlp": {"kind": "dense", "ff": 100}},
+                       {"type": "mamba2", "mixer": ss, "mlp": _vx_moe(3, 1, 40)}]}
+
+
+def _vx_c():
+    at = {"heads": 4, "kv_heads": 1, "dim": 64, "vdim": 64, "scale": 0.25, "rot": _vx_rot(500.0, 32, (16.0, 64, 4.0, 0.5))}
+    free = {"heads": 2, "kv_heads": 2, "dim": 128, "vdim": 32, "scale": 0.2}
+    de = {"heads": 2, "kv_heads": 1, "dim": 64, "vdim": 128, "conv": 4, "decay_rank": 32, "gate_rank": 16}
+    ss = {"heads": 4, "vdim": 64, "state": 128, "groups": 1, "norm_groups": 2, "conv": 4}
+    dense = {"kind": "dense", "ff": 256}
+    return {"architecture": "Vifirax", "vocab": 300, "width": 128, "norm": {"eps": 1e-6}, "logit_scale": 2.0,
+            "layers": [{"type": "channel_delta", "mixer": de, "mlp": dense},
+                       {"type": "attention", "mixer": at, "mlp": _vx_moe(8, 2, 64)},
+                       {"type": "mamba2", "mixer": ss, "mlp": dense},
+                       {"type": "attention", "mixer": dict(at, kv_from=1), "mlp": None},
+                       {"type": "attention", "mixer": free, "mlp": dense},
+                       {"type": "attention", "mixer": dict(at, kv_from=1), "mlp": _vx_moe(4, 3, 32)}]}
+
+
+def _vx_d():
+    at = {"heads": 6, "kv_heads": 2, "dim": 16, "vdim": 24, "scale": 0.7, "rot": _vx_rot(50.0, 16, (2.0, 32, 2.0, 1.0))}
+    ss = {"heads": 2, "vdim": 24, "state": 136, "groups": 1, "norm_groups": 3, "conv": 2}
+    de = {"heads": 1, "kv_heads": 1, "dim": 136, "vdim": 24, "conv": 5, "decay_rank": 3, "gate_rank": 9}
+    return {"architecture": "Vifirax", "vocab": 61, "width": 48, "norm": {"eps": 2e-6}, "logit_scale": 0.8,
+            "layers": [{"type": "attention", "mixer": at, "mlp": None},
+                       {"type": "attention", "mixer": dict(at, kv_from=0), "mlp": _vx_moe(4, 3, 16)},
+                       {"type": "mamba2", "mixer": ss, "mlp": {"kind": "dense", "ff": 80}},
+                       {"type": "attention", "mixer": dict(at, kv_from=0), "mlp": {"kind": "dense", "ff": 64}},
+                       {"type": "channel_delta", "mixer": de, "mlp": _vx_moe(7, 2, 8)}]}
+
+
+VIFIRAX = {"vx-a": _vx_a, "vx-b": _vx_b, "vx-c": _vx_c, "vx-d": _vx_d}
+
+
+def vifirax_tensors(raw: dict, seed: int):
+    """Random tensors for a Vifirax configuration, by name, in bfloat16 on the CPU: matrices N(0, gain^2 / inputs) with
+    gains that make every mechanism matter (sharp softmaxes, gates that open and close, routers that decide, decays
+    from fast to almost none), layer norm weights around 0 (they enter as 1 + w) and the mixers' plain ones around 1."""
+    import alice_llm_amd as alice
+    from alice_llm_amd.engine.model import CausalLM
+    from alice_llm_amd.parts import Precision
+    cfg = alice.config_from_dict(raw)
+    specs = CausalLM(cfg.plan(), Precision.of("float32"), "cpu").param_specs()
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, spec in specs.items():
+        shape = tuple(spec.shape)
+        r = torch.randn(shape, generator=g)
+        last = name.rsplit(".", 1)[-1]
+        if last == "A_log":
+            t = -2.0 + 1.5 * r                      # rates from a few thousandths to about one
+        elif last == "dt_bias":
+            t = 0.5 * r
+        elif last == "D":
+            t = r
+        elif last == "conv":
+            t = 0.6 * r
+        elif len(shape) == 1 and (last in ("norm1", "norm2") or name == "final.norm"):
+            t = 0.2 * r
+        elif len(shape) == 1:
+            t = 0.5 * r if last == "b" else 1.0 + 0.2 * r
+        elif name == "embed":
+            t = r * 0.5
+        else:
+            gain = 2.5 if last in ("q", "k", "g", "a2", "g2", "router", "b") else 1.0
+            t = r * gain / shape[1] ** 0.5
+        out[name] = t.to(torch.bfloat16)
+    return cfg, out
+
+
+def vifirax_pair(name: str, dtype: str, seed: int = 0, device="cuda"):
+    """(the package's model, the plain model) on the same tensors."""
+    from plain.vifirax_plain import PlainVifirax
+    raw = VIFIRAX[name]()
+    cfg, tensors = vifirax_tensors(raw, seed)
+    plain = PlainVifirax(raw, {k: v.double() for k, v in tensors.items()})
+    model = model_from_tensors(cfg, {k: v.to(device) for k, v in tensors.items()}, dtype)
+    return model, plain
+
+
+def vifirax_folder(name: str, seed: int = 0) -> str:
+    """A model folder (config.json without the widths of the narrow middles, which the tensors give; model.safetensors in
+    bfloat16) of a Vifirax test configuration."""
+    global _TMP
+    key = ("vifirax", name, seed)
+    if key not in _FOLDERS:
+        from safetensors.torch import save_file
+        if _TMP is None:
+            _TMP = tempfile.TemporaryDirectory(prefix="alice_tests_")
+        folder = os.path.join(_TMP.name, f"{name}-{seed}")
+        os.makedirs(folder, exist_ok=True)
+        raw = VIFIRAX[name]()
+        _, tensors = vifirax_tensors(raw, seed)
+        for l in raw["layers"]:
+            l["mixer"].pop("decay_rank", None)
+            l["mixer"].pop("gate_rank", None)
+        with open(os.path.join(folder, "config.json"), "w") as f:
+            json.dump(raw, f)
+        save_file({k: v.contiguous() for k, v in tensors.items()}, os.path.join(folder, "model.safetensors"))
+        _FOLDERS[key] = folder
+    return _FOLDERS[key]
