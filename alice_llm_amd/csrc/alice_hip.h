@@ -185,7 +185,9 @@ int alice_delta_prepare(float* qk, int qk_w, int k_col, int G, int d, float unit
 int alice_matrix_recurrence(const float* q, int q_w, int q_col, const float* k, int k_w, int k_col, const float* v, int v_w,
                             int v_col, const float* decay, int decay_per_row, const float* b, const float* skip, float* out,
                             const int* cu_seqlens, const int* slots, float* S, int n_seqs, int n_slots, int H, int qk_heads,
-                            int d, int dv, int delta, hipStream_t stream);
+                            int d, int dv, int delta, int columns, hipStream_t stream);
+// (columns: value columns a wave, 4, 8 or 16; 0: by the step's size, the rule of alice_matrix_recurrence_columns)
+int alice_matrix_recurrence_columns(int n_seqs, int H, int d, int dv);
 // Rows of `width` in `parts` equal parts, each RMS-normed and multiplied by a weight (w_shared: of a part's length);
 // gate_act 1: times silu(gate) before the norm, 2: times sigmoid(gate) after it, 0: no gate.
 int alice_norm_gate(const float* x, int width, int parts, const float* gate, int gate_w, int gate_col, int gate_act,

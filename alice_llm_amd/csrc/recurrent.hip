@@ -11,11 +11,12 @@
 // convolutions, the decays, step sizes and unit vectors are made with the full-precision functions, the state lives
 // in float32 rows of the cache, one per slot, and the read-out is left in float32 for the norm that follows.
 //
-// recurrence_kernel: one wave per (sequence, head, 16 value columns) walks through the sequence's tokens of the
+// recurrence_kernel: one wave per (sequence, head, CB value columns), four of them a block, walks through the sequence's tokens of the
 // step with its part of the state in registers: lane (rg, col) holds RPT neighbouring rows of one column, reads
 // them once and writes them once; a single token is the same walk of one step.  The tokens go through LDS TC at a
-// time; sums over the rows of a column meet by two lane exchanges (the four row groups of a column sit in one wave),
-// so the delta rule's two sums a token need no barrier.  Which rows belong to the sequence and which state row is
+// time, the next TC tokens' operands already on their way from memory; sums over the rows of a column meet by lane
+// exchanges inside a row of 16 lanes (the 64 / CB row groups of a column are neighbouring lanes), so the delta rule's
+// sum a token needs no barrier and no trip through LDS; the read-outs' sums are taken once per TC tokens.  CB is 16 where that fills the chip's SIMDs, else 8 or 4 (more waves, fewer rows a lane).  Which rows belong to the sequence and which state row is
 // its own are read on the device (cu_seqlens, slots), so a launch depends on sizes only.
 //
 // short_conv: y[t, c] = act(bias_c + sum_j w[c, j] x[t - (taps - 1) + j, c]) over the tokens of the token's own
@@ -130,17 +131,38 @@ struct RecurrenceArgs {
   int H, per, d, dv;
 };
 
-template <int RPT, int TC, bool DELTA>
-__global__ __launch_bounds__(64) void recurrence_kernel(RecurrenceArgs a) {
-  constexpr int CB = 16, RG = 4, DP = RG * RPT;
-  constexpr int NL = TC * DP / 64;
+// x plus the x of the lane that a DPP control names (lanes a fixed distance apart inside a row of 16)
+template <int CTRL>
+__device__ __forceinline__ float dpp_add(float x) {
+  return x + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xF, 0xF, true));
+}
+// The sum over the RG neighbouring lanes that hold one column's row groups (RG 4, 8 or 16, aligned): every one of them
+// gets it.  Lanes 1 and 2 apart inside a quad, then the other quad of the half row, then the other half of the row.
+template <int RG>
+__device__ __forceinline__ float sum_row_groups(float x) {
+  x = dpp_add<0xB1>(x);                    // quad_perm [1, 0, 3, 2]
+  x = dpp_add<0x4E>(x);                    // quad_perm [2, 3, 0, 1]
+  if (RG >= 8) x = dpp_add<0x141>(x);      // row_half_mirror
+  if (RG >= 16) x = dpp_add<0x140>(x);     // row_mirror
+  return x;
+}
+
+template <int CB, int RPT, int TC, int WPB, bool DELTA>
+__global__ __launch_bounds__(64 * WPB) void recurrence_kernel(RecurrenceArgs a) {
+  constexpr int RG = 64 / CB, DP = RG * RPT, NT = 64 * WPB, CBB = CB * WPB;
+  constexpr int NL = TC * DP / NT;
+  constexpr int NV = (TC * CBB + NT - 1) / NT;
+  static_assert(RPT % 4 == 0 && (TC * DP) % NT == 0 && TC <= 64 && (RG == 4 || RG == 8 || RG == 16), "rows are read four at a time");
   __shared__ __align__(16) float sq[TC][DP];
   __shared__ __align__(16) float sk[TC][DP];
   __shared__ __align__(16) float sa[TC][DP];
-  __shared__ float sv[TC][CB];
+  __shared__ float sv[TC][CBB];
   __shared__ float sb[TC];
-  const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, col = lane % CB, rg = lane / CB;
-  const int j = blockIdx.z * CB + col;
+  // the row groups of a column are neighbouring lanes, so that their sums meet without a trip through LDS; the waves of
+  // a block take neighbouring columns and share the tokens' q, k and decays
+  const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int col = wave * CB + lane / RG, rg = lane % RG;
+  const int j = blockIdx.z * CBB + col;
   const bool col_ok = j < a.dv;
   const int t0 = a.cu_seqlens[s], t1 = a.cu_seqlens[s + 1];
   if (t1 <= t0) return;
@@ -154,72 +176,97 @@ __global__ __launch_bounds__(64) void recurrence_kernel(RecurrenceArgs a) {
   }
   const int qk_head = h / a.per;
   const float skip = a.skip ? a.skip[h] : 0.f;
+  // what this thread fetches for TC tokens: element (t, r) = (idx / DP, idx % DP) of q, k and the decay; (t, c) of v; b of token `tid`
+  float pq[NL], pk[NL], pa[NL], pv[NV], pb = 0.f;
+  auto fetch = [&](int tc) {
+#pragma unroll
+    for (int n = 0; n < NL; ++n) {
+      const int idx = tid + n * NT, t = tc + idx / DP, r = idx % DP;
+      pq[n] = pk[n] = pa[n] = 0.f;
+      if (t < t1 && r < d) {
+        pq[n] = a.q[(size_t)t * a.q_w + a.q_col + qk_head * d + r];
+        pk[n] = a.k[(size_t)t * a.k_w + a.k_col + qk_head * d + r];
+        pa[n] = a.decay_per_row ? a.decay[((size_t)t * H + h) * d + r] : a.decay[(size_t)t * H + h];
+      }
+    }
+#pragma unroll
+    for (int n = 0; n < NV; ++n) {
+      const int idx = tid + n * NT, t = tc + idx / CBB, c = blockIdx.z * CBB + idx % CBB;
+      pv[n] = (idx < TC * CBB && t < t1 && c < dv) ? a.v[(size_t)t * a.v_w + a.v_col + h * dv + c] : 0.f;
+    }
+    pb = (tid < TC && tc + tid < t1) ? a.b[(size_t)(tc + tid) * H + h] : 0.f;
+  };
+  fetch(t0);
   for (int tc = t0; tc < t1; tc += TC) {
     const int n_tok = min(TC, t1 - tc);
     __syncthreads();                                   // the last tokens' operands have been read
 #pragma unroll
     for (int n = 0; n < NL; ++n) {
-      const int idx = lane + n * 64, tt = idx / DP, r = idx % DP;
-      const int t = tc + tt;
-      float xq = 0.f, xk = 0.f, xa = 0.f;
-      if (tt < n_tok && r < d) {
-        xq = a.q[(size_t)t * a.q_w + a.q_col + qk_head * d + r];
-        xk = a.k[(size_t)t * a.k_w + a.k_col + qk_head * d + r];
-        xa = a.decay_per_row ? a.decay[((size_t)t * H + h) * d + r] : a.decay[(size_t)t * H + h];
-      }
-      sq[tt][r] = xq;
-      sk[tt][r] = xk;
-      sa[tt][r] = xa;                                  // (rows beyond d hold zeros and stay zero)
+      const int idx = tid + n * NT;
+      sq[idx / DP][idx % DP] = pq[n];
+      sk[idx / DP][idx % DP] = pk[n];
+      sa[idx / DP][idx % DP] = pa[n];                  // (rows beyond d hold zeros and stay zero)
     }
-    for (int idx = lane; idx < TC * CB; idx += 64) {
-      const int tt = idx / CB, c = blockIdx.z * CB + idx % CB;
-      sv[tt][idx % CB] = (tt < n_tok && c < dv) ? a.v[(size_t)(tc + tt) * a.v_w + a.v_col + h * dv + c] : 0.f;
+#pragma unroll
+    for (int n = 0; n < NV; ++n) {
+      const int idx = tid + n * NT;
+      if (idx < TC * CBB) sv[idx / CBB][idx % CBB] = pv[n];
     }
-    if (lane < TC) sb[lane] = lane < n_tok ? a.b[(size_t)(tc + lane) * H + h] : 0.f;
+    if (tid < TC) sb[tid] = pb;
     __syncthreads();
-    for (int tt = 0; tt < n_tok; ++tt) {
-      const float vj = sv[tt][col], bt = sb[tt];
-      float u = bt * vj;
-      if (DELTA) {
-        float p = 0.f;
+    if (tc + TC < t1) fetch(tc + TC);                  // the next tokens' operands are on their way during the walk
+    float part[TC], vs[TC];                            // the lanes' shares of the read-outs meet once per TC tokens
+#pragma unroll
+    for (int tt = 0; tt < TC; ++tt) {
+      part[tt] = 0.f;
+      vs[tt] = 0.f;
+      if (tt < n_tok) {
+        const float vj = sv[tt][col], bt = sb[tt];
+        vs[tt] = vj;
+        float u = bt * vj;
+        float4 kk[RPT / 4];
+#pragma unroll
+        for (int i = 0; i < RPT; i += 4) kk[i / 4] = *reinterpret_cast<const float4*>(&sk[tt][rg * RPT + i]);
+        if (DELTA) {
+          float p0 = 0.f, p1 = 0.f, p2 = 0.f, p3 = 0.f;   // four sums side by side: no chain of dependent additions
+#pragma unroll
+          for (int i = 0; i < RPT; i += 4) {
+            const float4 aa = *reinterpret_cast<const float4*>(&sa[tt][rg * RPT + i]);
+            st[i] *= aa.x;      p0 = fmaf(st[i], kk[i / 4].x, p0);
+            st[i + 1] *= aa.y;  p1 = fmaf(st[i + 1], kk[i / 4].y, p1);
+            st[i + 2] *= aa.z;  p2 = fmaf(st[i + 2], kk[i / 4].z, p2);
+            st[i + 3] *= aa.w;  p3 = fmaf(st[i + 3], kk[i / 4].w, p3);
+          }
+          u = bt * (vj - sum_row_groups<RG>((p0 + p1) + (p2 + p3)));
+        }
+        float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
         for (int i = 0; i < RPT; i += 4) {
-          const float4 aa = *reinterpret_cast<const float4*>(&sa[tt][rg * RPT + i]);
-          const float4 kk = *reinterpret_cast<const float4*>(&sk[tt][rg * RPT + i]);
-          st[i] *= aa.x;      p = fmaf(st[i], kk.x, p);
-          st[i + 1] *= aa.y;  p = fmaf(st[i + 1], kk.y, p);
-          st[i + 2] *= aa.z;  p = fmaf(st[i + 2], kk.z, p);
-          st[i + 3] *= aa.w;  p = fmaf(st[i + 3], kk.w, p);
+          const float4 qq = *reinterpret_cast<const float4*>(&sq[tt][rg * RPT + i]);
+          if (DELTA) {
+            st[i] = fmaf(kk[i / 4].x, u, st[i]);
+            st[i + 1] = fmaf(kk[i / 4].y, u, st[i + 1]);
+            st[i + 2] = fmaf(kk[i / 4].z, u, st[i + 2]);
+            st[i + 3] = fmaf(kk[i / 4].w, u, st[i + 3]);
+          } else {
+            const float4 aa = *reinterpret_cast<const float4*>(&sa[tt][rg * RPT + i]);
+            st[i] = fmaf(aa.x, st[i], kk[i / 4].x * u);
+            st[i + 1] = fmaf(aa.y, st[i + 1], kk[i / 4].y * u);
+            st[i + 2] = fmaf(aa.z, st[i + 2], kk[i / 4].z * u);
+            st[i + 3] = fmaf(aa.w, st[i + 3], kk[i / 4].w * u);
+          }
+          o0 = fmaf(st[i], qq.x, o0);
+          o1 = fmaf(st[i + 1], qq.y, o1);
+          o2 = fmaf(st[i + 2], qq.z, o2);
+          o3 = fmaf(st[i + 3], qq.w, o3);
         }
-        p += __shfl_xor(p, CB, 64);
-        p += __shfl_xor(p, 2 * CB, 64);
-        u = bt * (vj - p);
+        part[tt] = (o0 + o1) + (o2 + o3);
       }
-      float o = 0.f;
+    }
 #pragma unroll
-      for (int i = 0; i < RPT; i += 4) {
-        const float4 kk = *reinterpret_cast<const float4*>(&sk[tt][rg * RPT + i]);
-        const float4 qq = *reinterpret_cast<const float4*>(&sq[tt][rg * RPT + i]);
-        if (DELTA) {
-          st[i] = fmaf(kk.x, u, st[i]);
-          st[i + 1] = fmaf(kk.y, u, st[i + 1]);
-          st[i + 2] = fmaf(kk.z, u, st[i + 2]);
-          st[i + 3] = fmaf(kk.w, u, st[i + 3]);
-        } else {
-          const float4 aa = *reinterpret_cast<const float4*>(&sa[tt][rg * RPT + i]);
-          st[i] = fmaf(aa.x, st[i], kk.x * u);
-          st[i + 1] = fmaf(aa.y, st[i + 1], kk.y * u);
-          st[i + 2] = fmaf(aa.z, st[i + 2], kk.z * u);
-          st[i + 3] = fmaf(aa.w, st[i + 3], kk.w * u);
-        }
-        o = fmaf(st[i], qq.x, o);
-        o = fmaf(st[i + 1], qq.y, o);
-        o = fmaf(st[i + 2], qq.z, o);
-        o = fmaf(st[i + 3], qq.w, o);
-      }
-      o += __shfl_xor(o, CB, 64);
-      o += __shfl_xor(o, 2 * CB, 64);
-      if (rg == 0 && col_ok) a.out[(size_t)(tc + tt) * H * dv + h * dv + j] = fmaf(skip, vj, o);
+    for (int tt = 0; tt < TC; ++tt) {
+      const float o = sum_row_groups<RG>(part[tt]);
+      if (tt < n_tok && rg == 0 && col_ok) a.out[(size_t)(tc + tt) * H * dv + h * dv + j] = fmaf(skip, vs[tt], o);
     }
   }
 #pragma unroll
@@ -307,29 +354,49 @@ extern "C" int alice_delta_prepare(float* qk, int qk_w, int k_col, int G, int d,
   return 0;
 }
 
+// Value columns a wave: 16 where (sequences x heads x columns) fill the chip's SIMDs, else 8 or 4: more waves, each with
+// fewer rows a lane (the rows of a column are then spread over 8 or 16 lanes).
+extern "C" int alice_matrix_recurrence_columns(int n_seqs, int H, int d, int dv) {
+  const long waves16 = (long)n_seqs * H * ceil_div(dv, 16);
+  return (waves16 >= 1024 || d <= 32) ? 16 : ((waves16 >= 512 || d <= 64) ? 8 : 4);
+}
+
 extern "C" int alice_matrix_recurrence(const float* q, int q_w, int q_col, const float* k, int k_w, int k_col, const float* v, int v_w,
                                        int v_col, const float* decay, int decay_per_row, const float* b, const float* skip, float* out,
                                        const int* cu_seqlens, const int* slots, float* S, int n_seqs, int n_slots, int H, int qk_heads,
-                                       int d, int dv, int delta, hipStream_t stream) {
+                                       int d, int dv, int delta, int columns, hipStream_t stream) {
   ALICE_CHECK(q && k && v && decay && b && out && cu_seqlens && slots && S, "matrix_recurrence: a pointer is missing");
   ALICE_CHECK(n_seqs >= 0 && n_slots >= 1 && H >= 1 && qk_heads >= 1 && H % qk_heads == 0 && d >= 1 && dv >= 1, "matrix_recurrence: bad sizes");
   ALICE_CHECK(d <= 256, "matrix_recurrence: key size %d is beyond 256, the range of this kernel", d);
   ALICE_CHECK(q_col >= 0 && k_col >= 0 && v_col >= 0 && q_col + qk_heads * d <= q_w && k_col + qk_heads * d <= k_w && v_col + H * dv <= v_w,
               "matrix_recurrence: the rows are too short for the heads");
-  ALICE_CHECK(H <= 65535 && ceil_div(dv, 16) <= 65535, "matrix_recurrence: too many heads for one launch");
+  ALICE_CHECK(H <= 65535 && ceil_div(dv, 16) <= 65535, "matrix_recurrence: too many heads or value columns for one launch");
   if (n_seqs == 0) return 0;
   RecurrenceArgs a{q, q_w, q_col, k, k_w, k_col, v, v_w, v_col, decay, decay_per_row, b, skip, out, cu_seqlens, slots, S, H, H / qk_heads, d, dv};
-  dim3 grid(n_seqs, H, ceil_div(dv, 16));
-#define GO(RPT, TC)                                                          \
-  do {                                                                       \
-    if (delta) recurrence_kernel<RPT, TC, true><<<grid, 64, 0, stream>>>(a); \
-    else recurrence_kernel<RPT, TC, false><<<grid, 64, 0, stream>>>(a);      \
+  int cb = columns ? columns : alice_matrix_recurrence_columns(n_seqs, H, d, dv);
+  ALICE_CHECK(cb == 16 || cb == 8 || cb == 4, "matrix_recurrence: %d value columns a wave are not built (4, 8, 16; 0: by the step's size)", columns);
+  if (d <= 32 || (cb == 4 && d <= 64)) cb = d <= 32 ? 16 : 8;      // (fewer than four rows a lane are not built)
+  constexpr int WPB = 4;                       // waves a block: they share the staged q, k and decays of a head's tokens
+  dim3 grid(n_seqs, H, ceil_div(dv, cb * WPB));
+#define GO(CB, RPT, TC)                                                                     \
+  do {                                                                                      \
+    if (delta) recurrence_kernel<CB, RPT, TC, WPB, true><<<grid, 64 * WPB, 0, stream>>>(a); \
+    else recurrence_kernel<CB, RPT, TC, WPB, false><<<grid, 64 * WPB, 0, stream>>>(a);      \
   } while (0)
-  if (d <= 16) GO(4, 16);
-  else if (d <= 32) GO(8, 16);
-  else if (d <= 64) GO(16, 16);
-  else if (d <= 128) GO(32, 8);
-  else GO(64, 8);
+  if (cb == 16) {
+    if (d <= 16) GO(16, 4, 16);
+    else if (d <= 32) GO(16, 8, 16);
+    else if (d <= 64) GO(16, 16, 16);
+    else if (d <= 128) GO(16, 32, 8);
+    else GO(16, 64, 8);
+  } else if (cb == 8) {
+    if (d <= 64) GO(8, 8, 16);
+    else if (d <= 128) GO(8, 16, 8);
+    else GO(8, 32, 8);
+  } else {
+    if (d <= 128) GO(4, 8, 8);
+    else GO(4, 16, 8);
+  }
 #undef GO
   ALICE_LAUNCH_CHECK();
   return 0;

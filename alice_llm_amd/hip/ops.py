@@ -69,7 +69,8 @@ def _declare(lib) -> None:
         "alice_short_conv": [P, I, I, I, I, P, P, P, P, I, P, P, P, I, I, P],
         "alice_ssm_prepare": [P, I, I, P, P, P, P, I, I, P],
         "alice_delta_prepare": [P, I, I, I, I, F, F, P, P, P, P, I, I, P, I, I, P],
-        "alice_matrix_recurrence": [P, I, I, P, I, I, P, I, I, P, I, P, P, P, P, P, P, I, I, I, I, I, I, I, P],
+        "alice_matrix_recurrence": [P, I, I, P, I, I, P, I, I, P, I, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
+        "alice_matrix_recurrence_columns": [I, I, I, I],
         "alice_norm_gate": [P, I, I, P, I, I, I, P, I, F, P, I, I, P],
         "alice_route_topk": [P, P, P, I, I, I, P],
         "alice_scale_columns": [P, I, P, P, I, I, I, I, P],
@@ -1043,13 +1044,21 @@ def delta_prepare(qk: torch.Tensor, k_col: int, z: torch.Tensor, dt_bias: torch.
           dt_bias.data_ptr(), a_log.data_ptr(), rows.data_ptr(), rows.shape[1], int(b_col), beta.data_ptr(), T, H, _stream())
 
 
+def recurrence_columns(n_seqs: int, heads: int, head_dim: int, value_head_dim: int) -> int:
+    """The value columns a wave that matrix_recurrence chooses for a step of this many sequences.  A caller whose steps
+    are also replayed from graphs recorded for a rounded-up number of sequences asks with that number and passes the answer
+    on, so that both kinds of step add in the same order."""
+    return library().alice_matrix_recurrence_columns(int(n_seqs), int(heads), int(head_dim), int(value_head_dim))
+
+
 def matrix_recurrence(q, q_col: int, k, k_col: int, v, v_col: int, decay: torch.Tensor, b: torch.Tensor, skip: Optional[torch.Tensor],
                       out: torch.Tensor, ctx, S: torch.Tensor, *, heads: int, qk_heads: int, head_dim: int, value_head_dim: int,
-                      delta: bool, decay_per_channel: bool) -> None:
+                      delta: bool, decay_per_channel: bool, columns_per_wave: int = 0) -> None:
     """The recurrence of a matrix state a head over a step (`ctx` gives cu_seqlens, slots, n_seqs), all float32:
     delta False: S = diag(a) S + k (b v)^T; True: S = diag(a) S, u = b (v - S^T k), S += k u^T; then o = S^T q (+ skip[h] v).
     q, k: rows with the heads' columns from q_col / k_col, shared by groups of heads / qk_heads heads; v: rows with
-    heads * dv columns from v_col; decay: [T, heads * d] (decay_per_channel) or [T, heads]; b: [T, heads]; S: [slots, heads, d, dv]; out: [T, heads * dv]."""
+    heads * dv columns from v_col; decay: [T, heads * d] (decay_per_channel) or [T, heads]; b: [T, heads]; S: [slots, heads, d, dv]; out: [T, heads * dv].
+    columns_per_wave: 0 lets the launcher choose by the step's size; 4, 8 or 16 fix the value columns a wave."""
     H, d, dv = heads, head_dim, value_head_dim
     T = out.shape[0]
     for t_, nm in ((q, "q"), (k, "k"), (v, "v")):
@@ -1069,7 +1078,7 @@ def matrix_recurrence(q, q_col: int, k, k_col: int, v, v_col: int, decay: torch.
     _call("alice_matrix_recurrence", q.data_ptr(), q.shape[1], int(q_col), k.data_ptr(), k.shape[1], int(k_col), v.data_ptr(),
           v.shape[1], int(v_col), decay.data_ptr(), int(per_row), b.data_ptr(), _opt(skip, "skip"), out.data_ptr(),
           ctx.cu_seqlens.data_ptr(), ctx.slots.data_ptr(), S.data_ptr(), int(ctx.n_seqs), int(n_slots), H, int(qk_heads), d, dv,
-          int(bool(delta)), _stream())
+          int(bool(delta)), int(columns_per_wave), _stream())
 
 
 def norm_gate(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor, *, parts: int, eps: float, weight_shared: bool,

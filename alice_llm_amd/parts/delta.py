@@ -132,7 +132,8 @@ class ChannelDeltaMixer(Part):
         o = torch.empty((T, self.vw), dtype=torch.float32, device=dev)
         ops.matrix_recurrence(conv, 0, conv, self.qk, conv, 2 * self.qk, z, beta, None, o, ctx, cache.state["S"],
                               heads=self.nH, qk_heads=self.nKV, head_dim=self.d, value_head_dim=self.P, delta=True,
-                              decay_per_channel=True)
+                              decay_per_channel=True,
+                              columns_per_wave=ops.recurrence_columns(getattr(ctx, "rounded_seqs", 0) or ctx.n_seqs, self.nH, self.d, self.P))
         out = torch.empty((T, self.vw), dtype=act, device=dev)
         ops.norm_gate(o, self.small[n["norm"]], out, parts=self.nH, eps=self.eps, weight_shared=True, gate=gate, gate_col=0,
                       gate_act="sigmoid")

@@ -99,7 +99,8 @@ class StateSpaceMixer(Part):
         b_col = self.inner
         ops.matrix_recurrence(conv, b_col + self.G * self.N, conv, b_col, conv, 0, decay, step, self.small[n["D"]], y, ctx,
                               cache.state["S"], heads=self.nH, qk_heads=self.G, head_dim=self.N, value_head_dim=self.P,
-                              delta=False, decay_per_channel=False)
+                              delta=False, decay_per_channel=False,
+                              columns_per_wave=ops.recurrence_columns(getattr(ctx, "rounded_seqs", 0) or ctx.n_seqs, self.nH, self.N, self.P))
         out = torch.empty((T, self.inner), dtype=self.precision.act, device=dev)
         ops.norm_gate(y, self.small[n["norm"]], out, parts=self.norm_groups, eps=self.eps, weight_shared=False,
                       gate=rows, gate_col=0, gate_act="silu")

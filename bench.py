@@ -15,6 +15,8 @@ of 6,000 tokens, past the window, at the 27B shape.
         instead of the above: the Telulorn design beside Novotar and Gemma 2 at equal layer sizes, in a line of its own
     python bench.py --pefitar w2048,w4096
         instead of the above: the Pefitar design beside Telulorn and Gemma 2 at equal layer sizes, in a line of its own
+    python bench.py --vifirax w2048,w4096
+        instead of the above: the Vifirax design beside Telulorn and Gemma 2 at equal layer sizes, in a line of its own
     python bench.py --novotar w2048,w4096
         instead of the above: prefill and decode throughput of the Novotar design at layer sizes of real models
         (random weights, a few layers), beside Gemma 2 at equal sizes; prints a line of its own
@@ -349,7 +351,27 @@ def pefitar_configs(size, vocab=32768, window=1024):
             "logit_softcap": 30.0, "layers": [lat, att, lat, att], "loop": {"start": 1, "stop": 3, "times": 2}}
 
 
-def novotar_bench(sizes, dtype, steps, warmup, with_telulorn=False, with_pefitar=False):
+def vifirax_configs(size, vocab=32768):
+    """A Vifirax configuration of six layers (attention, state space, delta rule, attention on the first layer's keys, state
+    space, delta rule) at the sizes of novotar_pair_configs: the same width and attention heads; every earlier key
+    visible; the state-space layers with an inner width of twice the model's in heads of 64 and a state of 128; the
+    delta-rule layers with the attention's heads and head size; feed-forwards in turn dense (the same size) and routed
+    (16 experts of a quarter of that size, 2 a token: half the dense layer's work a token, four times its weights)."""
+    z = NOVOTAR_SIZES[size]
+    dense = {"kind": "dense", "ff": z["ff"]}
+    moe = {"kind": "moe", "expert": {"ff": z["ff"] // 4}, "router": {"experts": 16, "top": 2}}
+    att = {"heads": z["heads"], "kv_heads": z["kv"], "dim": z["dim"], "vdim": z["dim"], "scale": z["dim"] ** -0.5,
+           "rot": {"base": 10000.0, "dims": z["dim"] // 2, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+    ssm = {"heads": 2 * z["width"] // 64, "vdim": 64, "state": 128, "groups": 1, "norm_groups": 1, "conv": 4}
+    dlt = {"heads": z["heads"], "kv_heads": z["heads"], "dim": z["dim"], "vdim": z["dim"], "conv": 4, "decay_rank": z["dim"],
+           "gate_rank": z["dim"]}
+    layers = [{"type": "attention", "mixer": att, "mlp": dense}, {"type": "mamba2", "mixer": ssm, "mlp": moe},
+              {"type": "channel_delta", "mixer": dlt, "mlp": dense}, {"type": "attention", "mixer": dict(att, kv_from=0), "mlp": moe},
+              {"type": "mamba2", "mixer": ssm, "mlp": dense}, {"type": "channel_delta", "mixer": dlt, "mlp": moe}]
+    return {"architecture": "Vifirax", "vocab": vocab, "width": z["width"], "norm": {"eps": 1e-6}, "logit_scale": 0.5, "layers": layers}
+
+
+def novotar_bench(sizes, dtype, steps, warmup, with_telulorn=False, with_pefitar=False, with_vifirax=False):
     out = {}
     for size in sizes:
         if size not in NOVOTAR_SIZES:
@@ -360,6 +382,8 @@ def novotar_bench(sizes, dtype, steps, warmup, with_telulorn=False, with_pefitar
             models.insert(0, ("telulorn", telulorn_configs(size)))
         if with_pefitar:
             models = [("pefitar", pefitar_configs(size)), ("telulorn", telulorn_configs(size)), models[-1]]
+        if with_vifirax:
+            models = [("vifirax", vifirax_configs(size)), ("telulorn", telulorn_configs(size)), models[-1]]
         for name, raw in models:
             run = Run(None, None, dtype, raw=raw)
             r = {"weights_gb": round(run.weight_bytes / 1e9, 3), "layer_runs": len(run.model.lm.plan.schedule)}
@@ -437,6 +461,8 @@ def main() -> int:
                     "equal sizes instead of the default workload, and print a line of its own")
     ap.add_argument("--pefitar", default="", help="sizes (w2048,w4096): measure the Pefitar design beside Telulorn and Gemma 2 at "
                     "equal layer sizes, in a line of its own")
+    ap.add_argument("--vifirax", default="", help="sizes (w2048,w4096): measure the Vifirax design beside Telulorn and Gemma 2 at "
+                    "equal layer sizes, in a line of its own")
     ap.add_argument("--no-peaks", action="store_true", help="skip the measurement of this GPU's own copy and matrix-product rates")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -445,6 +471,13 @@ def main() -> int:
 
     import torch
     torch.cuda.set_device(0)
+    if args.vifirax:
+        steps = min(args.steps, 64)
+        res = novotar_bench([x for x in args.vifirax.split(",") if x], args.dtype, steps, min(args.warmup, 5), with_vifirax=True)
+        print(json.dumps({"metric": "Vifirax beside Telulorn and Gemma 2 at equal layer sizes: prefill and decode, random weights",
+                          "unit": "tokens/s", "n_gpus": 1, "steps": steps, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+                          "data": "synthetic (uniform random token ids, random weights)", "sizes": res}), flush=True)
+        return 0
     if args.pefitar:
         steps = min(args.steps, 64)
         res = novotar_bench([x for x in args.pefitar.split(",") if x], args.dtype, steps, min(args.warmup, 5), with_pefitar=True)

@@ -510,6 +510,7 @@ def pefitar_folder(name: str, seed: int = 0) -> str:
 #    an attention layer with no rotation at all.
 # D: two layers that read the first layer's keys; key sizes of the recurrences beyond 128; five taps; three query heads a
 #    kv head; three norm parts; a single delta-rule head.
+# E: no attention at all (the cache holds no pages); a group a head and a norm part a head; two experts, both for every token.
 def _vx_rot(base, dims, scaling=None):
     rot = {"base": base, "dims": dims}
     if scaling is not None:
@@ -569,7 +570,16 @@ def _vx_d():
                        {"type": "channel_delta", "mixer": de, "mlp": _vx_moe(7, 2, 8)}]}
 
 
-VIFIRAX = {"vx-a": _vx_a, "vx-b": _vx_b, "vx-c": _vx_c, "vx-d": _vx_d}
+def _vx_e():
+    ss = {"heads": 8, "vdim": 8, "state": 16, "groups": 4, "norm_groups": 2, "conv": 3}
+    de = {"heads": 2, "kv_heads": 1, "dim": 32, "vdim": 40, "conv": 4, "decay_rank": 4, "gate_rank": 4}
+    return {"architecture": "Vifirax", "vocab": 83, "width": 40, "norm": {"eps": 1e-6}, "logit_scale": 1.5,
+            "layers": [{"type": "channel_delta", "mixer": de, "mlp": _vx_moe(2, 2, 24)},
+                       {"type": "mamba2", "mixer": ss, "mlp": None},
+                       {"type": "mamba2", "mixer": dict(ss, groups=8, norm_groups=8, conv=2), "mlp": {"kind": "dense", "ff": 56}}]}
+
+
+VIFIRAX = {"vx-a": _vx_a, "vx-b": _vx_b, "vx-c": _vx_c, "vx-d": _vx_d, "vx-e": _vx_e}
 
 
 def vifirax_tensors(raw: dict, seed: int):

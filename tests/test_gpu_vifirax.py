@@ -134,9 +134,11 @@ def test_short_convolution_over_pieces_with_carried_inputs(C, taps, col0, bias):
 
 
 @pytest.mark.parametrize("delta", [False, True])
+@pytest.mark.parametrize("cols", [0, 4, 8, 16])
 @pytest.mark.parametrize("H,G,d,dv", [(4, 2, 8, 16), (3, 3, 12, 20), (2, 1, 64, 128), (1, 1, 136, 24), (2, 2, 200, 7), (6, 3, 1, 1)])
-def test_matrix_recurrence_over_pieces_and_slots(delta, H, G, d, dv):
-    """Both recurrences against the plain scan, the state carried from step to step in the slots' rows."""
+def test_matrix_recurrence_over_pieces_and_slots(delta, cols, H, G, d, dv):
+    """Both recurrences against the plain scan, the state carried from step to step in the slots' rows; with the value
+    columns a wave left to the launcher and fixed at each of its choices."""
     data = {}
     for i, n in _TOTAL.items():
         q, k = rnd(n, G * d, seed=20 + i), rnd(n, G * d, seed=30 + i)
@@ -172,7 +174,8 @@ def test_matrix_recurrence_over_pieces_and_slots(delta, H, G, d, dv):
         q, k, v, decay, b = (cat(j) for j in range(5))
         out = torch.empty(q.shape[0], H * dv, device=DEV)
         ops.matrix_recurrence(q, 0, k, 0, v, 0, decay, b, None if skip is None else skip.to(DEV), out, _Ctx(lens, slots), S,
-                              heads=H, qk_heads=G, head_dim=d, value_head_dim=dv, delta=delta, decay_per_channel=delta)
+                              heads=H, qk_heads=G, head_dim=d, value_head_dim=dv, delta=delta, decay_per_channel=delta,
+                              columns_per_wave=cols)
         at = 0
         for i, (a, e) in zip(ids, spans):
             ref = refs[i][0][a:e].reshape(e - a, H * dv)
@@ -375,7 +378,8 @@ def test_far_key_and_the_one_in_the_denominator(dtype, H, G, d, dv, T):
     ops.attention_masked(qd, kp, vp, out, pos, seq, bt, max_position=T - 1, full_precision=dtype == "float32", gate=gd, **common)
     assert max_err(out, ref.reshape(T, H * dv)) < tol
     if ops.attention_tiled_supported(dt, d, dv):
-        for pieces in ([(0, T)], [(0, 2), (2, 63), (63, 66), (66, T - 9), (T - 9, T - 7), (T - 7, T)]):
+        cuts = sorted(c for c in {0, 2, 63, 66, T - 9, T - 7, T} if c <= T)
+        for pieces in ([(0, T)], list(zip(cuts[:-1], cuts[1:]))):
             st = _Step(pieces, T)
             o2 = torch.empty(len(st.rows), H * dv, dtype=dt, device=DEV)
             ops.attention_tiled(qd[st.rows], kp, vp, o2, st, bt.expand(st.n_seqs, -1).contiguous(), gate=gd[st.rows], **common)
@@ -501,7 +505,7 @@ def test_unequal_batch_against_each_alone_on_reused_slots(name, dtype):
     assert eng.cache.slots.n_free() == 4
 
 
-@pytest.mark.parametrize("name,dtype", [("vx-a", "float32"), ("vx-b", "bfloat16"), ("vx-c", "float32"), ("vx-d", "bfloat16")])
+@pytest.mark.parametrize("name,dtype", [("vx-a", "float32"), ("vx-b", "bfloat16"), ("vx-c", "float32"), ("vx-d", "bfloat16"), ("vx-e", "float32")])
 def test_long_decoding_from_the_first_token(name, dtype):
     model, plain = pair(name, dtype)
     toks = random_tokens(plain.config["vocab"], 330, 11)
