@@ -1,4 +1,4 @@
-"""alice-llm_amd: a small library for one MI355X (Gemma 2, Novotar, Telulorn and Pefitar): configuration and registry, safetensors
+"""alice-llm_amd: a small library for one MI355X (Gemma 2, Novotar, Telulorn, Pefitar and Vifirax): configuration and registry, safetensors
 weights, layers built from parts, a paged cache with slots, one step function, a generation loop
 with sampling, and hand-written HIP kernels for gfx950 in bfloat16 and in true 32-bit."""
 from .config import (ConfigError, Gemma2Config, NovotarConfig, PefitarConfig, TelulornConfig, VifiraxConfig, config_from_dict, load_config, register_architecture,

@@ -50,11 +50,11 @@ __global__ __launch_bounds__(64) void route_kernel(const float* __restrict__ z, 
 
 template <typename TI, typename TO>
 __global__ void scale_columns_kernel(const TI* __restrict__ x, const float* __restrict__ w, TO* __restrict__ y, long n, int E, int F) {
-  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  const long t = i / ((long)E * F);
-  const int e = (int)((i / F) % E);
-  store_f32(y, (size_t)i, load_f32(x, (size_t)i) * w[t * E + e]);
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+    const long t = i / ((long)E * F);
+    const int e = (int)((i / F) % E);
+    store_f32(y, (size_t)i, load_f32(x, (size_t)i) * w[t * E + e]);
+  }
 }
 
 }  // namespace
@@ -74,7 +74,8 @@ extern "C" int alice_scale_columns(const void* x, int x_dtype, const float* w, v
   ALICE_CHECK(T >= 0 && E >= 1 && F >= 1, "scale_columns: bad sizes");
   const long n = (long)T * E * F;
   if (n == 0) return 0;
-#define GO(TI, TO) scale_columns_kernel<TI, TO><<<ceil_div(n, 256), 256, 0, stream>>>((const TI*)x, w, (TO*)y, n, E, F)
+  const int blocks = (int)((n + 255) / 256 < (1L << 20) ? (n + 255) / 256 : (1L << 20));      // beyond that a thread takes several elements
+#define GO(TI, TO) scale_columns_kernel<TI, TO><<<blocks, 256, 0, stream>>>((const TI*)x, w, (TO*)y, n, E, F)
   if (x_dtype == DT_F32 && y_dtype == DT_F32) GO(float, float);
   else if (x_dtype == DT_F32) GO(float, bf16_t);
   else if (y_dtype == DT_F32) GO(bf16_t, float);

@@ -19,6 +19,7 @@ from .base import FEED_FORWARDS, ParamSpec, Part, Precision
 from .linear import Linear
 
 _GATED = {"gelu_tanh": 0.0, "silu": ops.GATED_SILU}
+MIDDLE_ELEMENTS = 1 << 28      # the most middle activations (tokens x experts x their width) that a step holds at a time
 
 
 @FEED_FORWARDS.register("expert_mlp")
@@ -83,7 +84,16 @@ class ExpertMLP(Part):
         logits = self.router(x, torch.float32)
         weights = torch.empty((T, self.E), dtype=torch.float32, device=dev)
         ops.route_topk(logits, self.bias, weights, self.top)
+        rows = max(1, MIDDLE_ELEMENTS // (self.E * self.F))
+        if T <= rows:
+            return self._experts(x, weights, True)
+        out = torch.empty((T, self.H), dtype=torch.float32, device=dev)      # a long step: the tokens in runs, so that the middle stays small
+        for a in range(0, T, rows):
+            out[a:a + rows] = self._experts(x[a:a + rows], weights[a:a + rows], False)
+        return out
+
+    def _experts(self, x, weights, allow_partials: bool) -> torch.Tensor:
         mid = self.gate_up(x, torch.float32)                 # every expert's middle activations, not yet rounded
-        scaled = torch.empty((T, self.E * self.F), dtype=self.precision.act, device=dev)
+        scaled = torch.empty(mid.shape, dtype=self.precision.act, device=mid.device)
         ops.scale_columns(mid, weights, scaled)
-        return self.down(scaled, torch.float32, allow_partials=True)
+        return self.down(scaled, torch.float32, allow_partials=allow_partials)
