@@ -196,6 +196,10 @@ int alice_norm_gate(const float* x, int width, int parts, const float* gate, int
 // zero elsewhere; and y[t, e F + j] = x[t, e F + j] w[t, e].  See experts.hip.
 int alice_route_topk(const float* z, const float* bias, float* w, int T, int E, int top, hipStream_t stream);
 int alice_scale_columns(const void* x, int x_dtype, const float* w, void* y, int y_dtype, int T, int E, int F, hipStream_t stream);
+// The routed feed-forward by grouped products over (token, expert) pairs in expert order (bfloat16, fragment layouts).
+long alice_expert_rows(int T, int E, int top);
+int alice_expert_products(const void* x, const float* weights, const void* gate_up, const void* down, float* y, int* ints,
+                          void* mid, float* rows, int T, int W, int F, int E, int top, float epi, hipStream_t stream);
 // Latent attention (latent.hip): the cache row of a token is [latent (kv_rank) | rotated key part (rot_dim)], one kv head,
 // row-major pages; the first kv_rank dimensions of a row are also its value.
 int alice_latent_prepare(const float* rows, int row_width, int q_rank, int kv_rank, int rot_dim, const float* w_q,

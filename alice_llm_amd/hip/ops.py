@@ -74,6 +74,7 @@ def _declare(lib) -> None:
         "alice_norm_gate": [P, I, I, P, I, I, I, P, I, F, P, I, I, P],
         "alice_route_topk": [P, P, P, I, I, I, P],
         "alice_scale_columns": [P, I, P, P, I, I, I, I, P],
+        "alice_expert_products": [P, P, P, P, P, P, P, P, I, I, I, I, I, F, P],
         "alice_add_rows": [P, P, P, I, I, P],
         "alice_latent_prepare": [P, I, I, I, I, P, P, F, P, P, P, P, P, I, I, I, P, P, I, I, P],
         "alice_heads_linear": [P, I, L, I, P, I, P, I, L, I, I, I, I, I, I, P, P, P, P],
@@ -101,6 +102,8 @@ def _declare(lib) -> None:
     lib.alice_attention_split_workspace.restype = L
     lib.alice_mlstm_chunks_workspace.argtypes = [I, I, I, I, I, I]
     lib.alice_mlstm_chunks_workspace.restype = L
+    lib.alice_expert_rows.argtypes = [I, I, I]
+    lib.alice_expert_rows.restype = L
 
 
 def _open(path: str):
@@ -1121,6 +1124,34 @@ def scale_columns(x: torch.Tensor, weights: torch.Tensor, out: torch.Tensor) -> 
     _dev(out, "out", None, tuple(x.shape))
     _call("alice_scale_columns", x.data_ptr(), dtype_code(x.dtype), weights.data_ptr(), out.data_ptr(), dtype_code(out.dtype),
           T, E, x.shape[1] // E, _stream())
+
+
+def expert_products_supported(dtype: torch.dtype, width: int, expert_width: int) -> bool:
+    """Whether expert_products takes these operands: bfloat16, a width that is a multiple of 8 and experts of a multiple of 32."""
+    return dtype == torch.bfloat16 and width >= 8 and width % 8 == 0 and expert_width >= 32 and expert_width % 32 == 0
+
+
+def expert_products(x: torch.Tensor, weights: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, y: torch.Tensor, *,
+                    expert_width: int, top: int, epi_param: float) -> None:
+    """The routed feed-forward by grouped products: y[t] = sum over the experts e that token t uses (weights[t, e] > 0) of
+    weights[t, e] * down_e(act(gate_e x[t]) * (up_e x[t])).  x: bfloat16 [T, W]; weights: float32 [T, E]; gate_up, down: the
+    fragment layouts of [all gates; all ups] ([2 E F, W]) and of the down matrices side by side ([W, E F]); y: float32
+    [T, W].  The (token, expert) pairs are put in expert order on the device; only the chosen experts are read."""
+    T, W = x.shape
+    E, F = weights.shape[1], int(expert_width)
+    if not expert_products_supported(x.dtype, W, F):
+        raise HipLibraryError("expert_products: bfloat16, a width that is a multiple of 8 and experts of a multiple of 32")
+    _dev(x, "x", torch.bfloat16)
+    _dev(weights, "weights", torch.float32, (T, E))
+    _dev(gate_up, "gate_up", torch.bfloat16, (frag_rows(2 * E * F) * (-(-W // 32) * 32),))
+    _dev(down, "down", torch.bfloat16, (frag_rows(W) * (-(-(E * F) // 32) * 32),))
+    _dev(y, "y", torch.float32, (T, W))
+    R = library().alice_expert_rows(T, E, int(top))
+    ints = torch.empty((2 * R + R // 64 + T * top,), dtype=torch.int32, device=x.device)
+    mid = torch.empty((R, F), dtype=torch.bfloat16, device=x.device)
+    rows = torch.empty((R, W), dtype=torch.float32, device=x.device)
+    _call("alice_expert_products", x.data_ptr(), weights.data_ptr(), gate_up.data_ptr(), down.data_ptr(), y.data_ptr(),
+          ints.data_ptr(), mid.data_ptr(), rows.data_ptr(), T, W, F, E, int(top), float(epi_param), _stream())
 
 
 def fragment_layout_supported(rows: int, k_in: int, epilogue: int) -> bool:

@@ -4,9 +4,12 @@ Router logits z = R h + r in 32-bit; the `top` best-scoring experts serve the to
 wins) and are mixed by a softmax restricted to those `top` logits: y = sum_e w_e down_e(act(gate_e h) * (up_e h)).  Tensors: "router", "router.b", and "e<i>.gate", "e<i>.up", "e<i>.down" for every expert.
 
 The experts' gate and up matrices are stacked into one matrix at load, and their down matrices side by side into
-another: one gated product gives every expert's middle activations, each is multiplied by its expert's weight of
-that token (zero where the token does not use the expert), and one down projection over all of them is the weighted
-sum.  Every kernel's launch depends on sizes only, never on which experts the tokens chose.
+another.  Steps of few tokens, the 32-bit path and sizes that suit no tile: one gated product gives every expert's
+middle activations, each is multiplied by its expert's weight of that token (zero where the token does not use the
+expert), and one down projection over all of them is the weighted sum.  Steps of many tokens in bfloat16: the (token,
+expert) pairs are put in expert order on the device and each pair meets its own expert's matrices only (grouped
+products over the same stacked matrices).  Every kernel's launch depends on sizes only, never on which experts the
+tokens chose.
 """
 from __future__ import annotations
 
@@ -19,6 +22,7 @@ from .base import FEED_FORWARDS, ParamSpec, Part, Precision
 from .linear import Linear
 
 _GATED = {"gelu_tanh": 0.0, "silu": ops.GATED_SILU}
+GROUPED_FROM_TOKENS = 64       # steps of this many tokens and more take the grouped products (bfloat16, sizes that suit the tiles)
 MIDDLE_ELEMENTS = 1 << 28      # the most middle activations (tokens x experts x their width) that a step holds at a time
 
 
@@ -84,6 +88,13 @@ class ExpertMLP(Part):
         logits = self.router(x, torch.float32)
         weights = torch.empty((T, self.E), dtype=torch.float32, device=dev)
         ops.route_topk(logits, self.bias, weights, self.top)
+        if (T >= GROUPED_FROM_TOKENS and self.gate_up.layout == ops.LAYOUT_FRAG16 and self.down.layout == ops.LAYOUT_FRAG16
+                and ops.expert_products_supported(x.dtype, self.H, self.F)):
+            # enough tokens that the experts' products pay: each (token, expert) pair meets its own expert only
+            out = torch.empty((T, self.H), dtype=torch.float32, device=dev)
+            ops.expert_products(x, weights, self.gate_up.weight, self.down.weight, out, expert_width=self.F, top=self.top,
+                                epi_param=self.gate_up.epi_param)
+            return out
         rows = max(1, MIDDLE_ELEMENTS // (self.E * self.F))
         if T <= rows:
             return self._experts(x, weights, True)

@@ -248,7 +248,8 @@ def test_router_takes_the_largest_and_weights_them_by_their_own_softmax(T, E, to
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("T,W,F,E,top", [(5, 64, 24, 6, 2), (70, 72, 18, 5, 5), (130, 128, 64, 8, 2), (33, 48, 7, 3, 1)])
+@pytest.mark.parametrize("T,W,F,E,top", [(5, 64, 24, 6, 2), (70, 72, 18, 5, 5), (130, 128, 64, 8, 2), (33, 48, 7, 3, 1), (64, 40, 32, 4, 1),
+                                         (300, 256, 96, 16, 3), (1000, 72, 64, 3, 3), (257, 136, 160, 33, 4)])
 def test_routed_feed_forward(dtype, T, W, F, E, top):
     p = Precision.of(dtype)
     ff = FEED_FORWARDS.get("expert_mlp")(p, hidden_size=W, intermediate_size=F, experts=E, top=top, activation="silu")
