@@ -262,10 +262,16 @@ def test_routed_feed_forward(dtype, T, W, F, E, top):
         ff.assign(n, t)
     ff.finalize()
     x = rnd(T, W, seed=99).to(torch.bfloat16)                  # the router sees the same numbers on both paths
-    out = ff.forward(x.to(p.act).to(DEV), None)
-    out = out.sum(0) if out.dim() == 3 else out
     ref = P.routed_ff(x.double(), {k: v.double().cpu() for k, v in ws.items()}, {"router": {"experts": E, "top": top}})
-    assert max_err(out, ref) < (2e-5 if dtype == "float32" else 3e-2) * max(1.0, float(ref.abs().max()))
+    from alice_llm_amd.parts import experts
+    kept = experts.GROUPED_FROM_TOKENS
+    try:
+        for experts.GROUPED_FROM_TOKENS in (1, 10 ** 9, kept):  # the grouped products wherever they apply, never, and the part's own choice
+            out = ff.forward(x.to(p.act).to(DEV), None)
+            out = out.sum(0) if out.dim() == 3 else out
+            assert max_err(out, ref) < (2e-5 if dtype == "float32" else 3e-2) * max(1.0, float(ref.abs().max())), experts.GROUPED_FROM_TOKENS
+    finally:
+        experts.GROUPED_FROM_TOKENS = kept
     with pytest.raises(ValueError, match="top"):
         FEED_FORWARDS.get("expert_mlp")(p, hidden_size=W, intermediate_size=F, experts=E, top=E + 1)
 
