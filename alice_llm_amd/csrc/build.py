@@ -101,17 +101,25 @@ def build(verbose: bool = True) -> str:
     objs = {s: os.path.join(obj_dir, f"{s[:-4]}.{os.getpid()}.o") for s in srcs}
     t0 = time.time()
     workers = max(1, min(len(srcs), int(os.environ.get("MAX_JOBS", "0")) or (os.cpu_count() or 4), 16))
-    with cf.ThreadPoolExecutor(workers) as pool:
-        futs = {pool.submit(_compile, hipcc, s, o, digest): s for s, o in objs.items()}
-        pending = set(futs)
-        while pending:
-            done, pending = cf.wait(pending, timeout=15, return_when=cf.FIRST_COMPLETED)
-            for f in done:
-                dt = f.result()
-                if verbose:
-                    _say(f"  {futs[f]} compiled in {dt:.0f} s")
-            if pending and verbose and not done:
-                _say(f"  still compiling {len(pending)} sources ({time.time() - t0:.0f} s)")
+    try:
+        with cf.ThreadPoolExecutor(workers) as pool:
+            futs = {pool.submit(_compile, hipcc, s, o, digest): s for s, o in objs.items()}
+            pending = set(futs)
+            while pending:
+                done, pending = cf.wait(pending, timeout=15, return_when=cf.FIRST_COMPLETED)
+                for f in done:
+                    dt = f.result()
+                    if verbose:
+                        _say(f"  {futs[f]} compiled in {dt:.0f} s")
+                if pending and verbose and not done:
+                    _say(f"  still compiling {len(pending)} sources ({time.time() - t0:.0f} s)")
+    except BaseException:
+        for o in objs.values():                    # a source that does not compile leaves no objects of the others behind
+            try:
+                os.remove(o)
+            except OSError:
+                pass
+        raise
     lib = os.path.join(out_dir, LIB_NAME)
     tmp = lib + f".tmp{os.getpid()}"
     r = subprocess.run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", tmp, *objs.values()],
